@@ -1,0 +1,102 @@
+/*
+ * C ABI of libpathsig_hip.so: signature / log-signature operators for AMD MI355X (gfx950).
+ *
+ * The four compute entry points are what a host binding of the reference's four operators calls
+ * (schemas in src/pathsig/bindings.cpp:9-63 of tobiasny12/pathsig).  All pointers are raw device or
+ * host addresses, all sizes are plain integers, nothing here depends on torch.
+ *
+ * Conventions
+ *   - dtype: PATHSIG_F32 or PATHSIG_F64; every floating buffer of one call has that type.
+ *   - device buffers are dense row-major and must not overlap; the library never allocates, frees,
+ *     or synchronises: scratch memory is passed in as `workspace` (size from the matching
+ *     *_workspace function; contents need not be initialised) and all work is enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL is the default stream).
+ *   - level_sizes is a HOST array with depth+1 entries (entry 0 unused) or NULL for the dense
+ *     signature.  A level whose size equals d^k is dense (all words, lexicographic); any other level
+ *     takes its words from encoded_words, a DEVICE int64 array with the base-d codes (first letter
+ *     most significant) of the non-dense levels concatenated in level order.
+ *   - windows is a DEVICE int32 array of W [start, end) pairs over point indices, or NULL.  Windows
+ *     are clamped to [0, L]; a window with fewer than two points yields zeros.
+ *   - return value: PATHSIG_OK or a negative error code; pathsig_last_error() gives the message of
+ *     the last failure on the calling thread.
+ */
+#ifndef PATHSIG_HIP_H
+#define PATHSIG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PATHSIG_F32 0
+#define PATHSIG_F64 1
+
+#define PATHSIG_OK 0
+#define PATHSIG_ERR_ARGUMENT (-1)    /* null pointer, bad dtype, depth outside 1..12, L < 2, ... */
+#define PATHSIG_ERR_UNSUPPORTED (-2) /* a size the kernels cannot handle */
+#define PATHSIG_ERR_WORKSPACE (-3)   /* workspace missing or too small */
+#define PATHSIG_ERR_LAUNCH (-4)      /* the HIP runtime rejected a launch */
+
+#define PATHSIG_MAX_DEPTH 12
+
+/* Library ABI version (bumped when a signature below changes). */
+int pathsig_abi_version(void);
+
+/* Message of the last error on this thread ("" if none). */
+const char *pathsig_last_error(void);
+
+/*
+ * Signature forward.  Replaces computeSignature (src/pathsig/forward/sig_launch.cu:75-225, op
+ * `pathsig::compute_signature`, src/pathsig/bindings.cpp:9-20).
+ *   path [B, L, d] -> sig [B, S] (windows == NULL) or [B, W, S];  S = sum of the level sizes.
+ */
+size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                                     const int64_t *level_sizes, int64_t W);
+int pathsig_sig_forward(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                        const int64_t *level_sizes, const int64_t *encoded_words, int64_t n_encoded,
+                        const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
+/*
+ * Signature backward: dL/dpath from dL/dsig.  Replaces signature_backward
+ * (src/pathsig/backward/sig_backward_launch.cu:83-303, op `pathsig::signature_backward`,
+ * src/pathsig/bindings.cpp:23-36).  `sig` is the forward output for the same arguments.
+ *   path [B, L, d], sig and grad_sig [B, (W,) S] -> grad_path [B, L, d].
+ * Gradients of overlapping windows add.
+ */
+size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                                      const int64_t *level_sizes, int64_t W);
+int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                         int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                         const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Signature -> log-signature on the hybrid layout (levels 1..depth-1 dense, level `depth` with
+ * `top_size` columns whose codes are `top_words`, a DEVICE int64 array, or NULL when the top level
+ * is dense).  Replaces sig_to_logsig (src/pathsig/forward/sig_launch.cu:230-339, op
+ * `pathsig::sig_to_logsig`, src/pathsig/bindings.cpp:39-49).
+ *   sig [rows, S] -> logsig [rows, S] and the power cache P [rows, S * depth] with
+ *   P[idx * depth + (m - 1)] = level-|w| part of (S - 1)^(x)m at word idx, 0 for m > |w|.
+ * Every element of logsig and P is written.
+ */
+int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, int64_t rows, int64_t d, int depth,
+                           int64_t top_size, const int64_t *top_words, void *stream);
+
+/*
+ * Adjoint of the above: dL/dsig from dL/dlogsig.  Replaces logsig_backward
+ * (src/pathsig/backward/sig_backward_launch.cu:307-460, op `pathsig::logsig_backward`,
+ * src/pathsig/bindings.cpp:52-63).
+ *   sig, grad_logsig [rows, S], P [rows, S * depth] -> grad_sig [rows, S].
+ */
+size_t pathsig_logsig_backward_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size);
+int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_logsig, void *grad_sig, int dtype,
+                            int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PATHSIG_HIP_H */

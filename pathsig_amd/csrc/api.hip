@@ -1,0 +1,361 @@
+// extern "C" entry points of libpathsig_hip.so: argument checks, level plans, kernel selection.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.hpp"
+#include "dense.hpp"
+
+namespace psig {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+namespace {
+
+constexpr int kWordsBlock = 256;
+
+size_t elem_size(int dtype) { return dtype == PATHSIG_F64 ? sizeof(double) : sizeof(float); }
+
+size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
+
+// d^k with overflow detection (returns -1 when it does not fit 62 bits)
+int64_t checked_pow(int64_t d, int k) {
+    int64_t r = 1;
+    for (int i = 0; i < k; ++i) {
+        if (r > (int64_t(1) << 62) / d) return -1;
+        r *= d;
+    }
+    return r;
+}
+
+int check_common(int dtype, int64_t B, int64_t L, int64_t d, int depth) {
+    if (dtype != PATHSIG_F32 && dtype != PATHSIG_F64) {
+        set_error("dtype must be PATHSIG_F32 or PATHSIG_F64 (got %d)", dtype);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (depth < 1 || depth > kMaxDepth) {
+        set_error("depth must be in [1,12] (got %d)", depth);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (B < 0 || d < 1) {
+        set_error("path must be [B,L,d] with B >= 0 and d >= 1 (got B=%lld d=%lld)", (long long)B, (long long)d);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (L < 2) {
+        set_error("path must have at least 2 time steps (got %lld)", (long long)L);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (d * (int64_t)elem_size(dtype) > 8192) {
+        set_error("path dimension %lld is beyond what the kernels stage in LDS", (long long)d);
+        return PATHSIG_ERR_UNSUPPORTED;
+    }
+    return PATHSIG_OK;
+}
+
+// Builds the per-level plan; returns PATHSIG_OK or an error.  *all_dense is set when every level is full.
+int build_plan(int64_t d, int depth, const int64_t *level_sizes, int64_t n_encoded, bool have_codes, LevelPlan *plan,
+               bool *all_dense) {
+    std::memset(plan, 0, sizeof(*plan));
+    plan->depth = depth;
+    int64_t out = 0, enc = 0, blocks = 0;
+    bool saved_ok = true;  // every level so far is dense: prefixes can be read from the saved signature
+    *all_dense = true;
+    for (int k = 1; k <= depth; ++k) {
+        const int64_t width = checked_pow(d, k);
+        int64_t size = width;
+        if (level_sizes) size = level_sizes[k];
+        if (size < 0) {
+            set_error("level_sizes[%d] is negative", k);
+            return PATHSIG_ERR_ARGUMENT;
+        }
+        if (!level_sizes && width < 0) {
+            set_error("d^%d does not fit 64 bits", k);
+            return PATHSIG_ERR_UNSUPPORTED;
+        }
+        const bool dense = (size == width);
+        plan->size[k] = size;
+        plan->out_off[k] = out;
+        plan->code_off[k] = dense ? -1 : enc;
+        plan->from_saved[k] = saved_ok ? 1 : 0;
+        plan->block_begin[k] = blocks;
+        if (!dense) {
+            enc += size;
+            *all_dense = false;
+            saved_ok = false;
+        }
+        out += size;
+        blocks += (size + kWordsBlock - 1) / kWordsBlock;
+    }
+    plan->block_begin[depth + 1] = blocks;
+    plan->sig_size = out;
+    if (enc > 0 && !have_codes) {
+        set_error("encoded_words is NULL but %lld word codes are needed", (long long)enc);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (enc > n_encoded) {
+        set_error("encoded_words holds %lld codes but the level sizes need %lld", (long long)n_encoded, (long long)enc);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    return PATHSIG_OK;
+}
+
+int check_grid(const LevelPlan &plan, int64_t rows) {
+    const int64_t per_row = plan.block_begin[plan.depth + 1];
+    if (per_row > 0 && rows > (int64_t(1) << 31) / per_row - 1) {
+        set_error("problem too large for one launch (%lld blocks per row x %lld rows)", (long long)per_row,
+                  (long long)rows);
+        return PATHSIG_ERR_UNSUPPORTED;
+    }
+    return PATHSIG_OK;
+}
+
+int launch_failed(hipError_t e, const char *what) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return PATHSIG_ERR_LAUNCH;
+}
+
+template <typename T>
+int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                  const int64_t *codes, int64_t n_encoded, const int32_t *windows, int64_t W, void *workspace,
+                  size_t workspace_bytes, hipStream_t stream) {
+    LevelPlan plan;
+    bool all_dense;
+    int rc = build_plan(d, depth, level_sizes, n_encoded, codes != nullptr, &plan, &all_dense);
+    if (rc != PATHSIG_OK) return rc;
+    SigShape shape{B, L, d, windows ? W : 1, windows};
+    if (B == 0 || shape.W == 0 || plan.sig_size == 0) return PATHSIG_OK;
+    rc = check_grid(plan, B * shape.W);
+    if (rc != PATHSIG_OK) return rc;
+    const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
+    if (dc.usable) {
+        if (workspace_bytes < dc.forward_workspace || (dc.forward_workspace && !workspace)) {
+            set_error("workspace too small: need %zu bytes, got %zu", dc.forward_workspace, workspace_bytes);
+            return PATHSIG_ERR_WORKSPACE;
+        }
+        hipError_t e = launch_dense_forward<T>((const T *)path, (T *)sig, shape, plan, codes, dc, workspace, stream);
+        if (e != hipSuccess) return launch_failed(e, "dense forward launch");
+        return PATHSIG_OK;
+    }
+    hipError_t e = launch_words_forward<T>((const T *)path, (T *)sig, shape, plan, codes, stream);
+    if (e != hipSuccess) return launch_failed(e, "forward launch");
+    return PATHSIG_OK;
+}
+
+template <typename T>
+int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void *grad_path, int64_t B, int64_t L,
+                   int64_t d, int depth, const int64_t *level_sizes, const int64_t *codes, int64_t n_encoded,
+                   const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    LevelPlan plan;
+    bool all_dense;
+    int rc = build_plan(d, depth, level_sizes, n_encoded, codes != nullptr, &plan, &all_dense);
+    if (rc != PATHSIG_OK) return rc;
+    SigShape shape{B, L, d, windows ? W : 1, windows};
+    if (B == 0) return PATHSIG_OK;
+    rc = check_grid(plan, B * shape.W);
+    if (rc != PATHSIG_OK) return rc;
+    const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
+    const size_t inc_bytes = align_up((size_t)(B * (L - 1) * d) * sizeof(T));
+    const size_t need = inc_bytes + (dc.usable ? dc.backward_workspace : 0);
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    T *ginc = (T *)workspace;
+    hipError_t e;
+    if (dc.usable) {
+        void *extra = (unsigned char *)workspace + inc_bytes;
+        e = launch_dense_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan, codes, dc,
+                                     extra, stream);
+        if (e != hipSuccess) return launch_failed(e, "dense backward launch");
+    } else {
+        e = launch_fill_zero<T>(ginc, B * (L - 1) * d, stream);
+        if (e != hipSuccess) return launch_failed(e, "fill launch");
+        if (shape.W > 0 && plan.sig_size > 0) {
+            e = launch_words_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan, codes,
+                                         stream);
+            if (e != hipSuccess) return launch_failed(e, "backward launch");
+        }
+    }
+    e = launch_increments_to_path<T>(ginc, (T *)grad_path, B, L, d, stream);
+    if (e != hipSuccess) return launch_failed(e, "path-gradient launch");
+    return PATHSIG_OK;
+}
+
+int check_logsig(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
+    if (dtype != PATHSIG_F32 && dtype != PATHSIG_F64) {
+        set_error("dtype must be PATHSIG_F32 or PATHSIG_F64 (got %d)", dtype);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (depth < 1 || depth > kMaxDepth) {
+        set_error("depth must be in [1,12] (got %d)", depth);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (d < 1 || rows < 0 || top_size < 0) {
+        set_error("d must be >= 1, rows and top_size >= 0");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (checked_pow(d, depth) < 0) {
+        set_error("d^depth does not fit 64 bits");
+        return PATHSIG_ERR_UNSUPPORTED;
+    }
+    if (rows >= (int64_t(1) << 31)) {
+        set_error("too many rows for one launch");
+        return PATHSIG_ERR_UNSUPPORTED;
+    }
+    return PATHSIG_OK;
+}
+
+int64_t lower_columns(int64_t d, int depth) {
+    int64_t acc = 0, width = 1;
+    for (int k = 1; k < depth; ++k) {
+        width *= d;
+        acc += width;
+    }
+    return acc;
+}
+
+}  // namespace
+}  // namespace psig
+
+using namespace psig;
+
+extern "C" {
+
+int pathsig_abi_version(void) { return 1; }
+
+const char *pathsig_last_error(void) { return g_error; }
+
+size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                                     const int64_t *level_sizes, int64_t W) {
+    if (check_common(dtype, B, L, d, depth) != PATHSIG_OK) return 0;
+    LevelPlan plan;
+    bool all_dense;
+    if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
+    const DenseChoice dc =
+        dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
+    return dc.usable ? dc.forward_workspace : 0;
+}
+
+int pathsig_sig_forward(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                        const int64_t *level_sizes, const int64_t *encoded_words, int64_t n_encoded,
+                        const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = check_common(dtype, B, L, d, depth);
+    if (rc != PATHSIG_OK) return rc;
+    if (B > 0 && (!path || !sig)) {
+        set_error("path and sig must not be NULL");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (windows && W < 0) {
+        set_error("W must be >= 0");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (dtype == PATHSIG_F32)
+        return sig_forward_t<float>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W,
+                                    workspace, workspace_bytes, (hipStream_t)stream);
+    return sig_forward_t<double>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W,
+                                 workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                                      const int64_t *level_sizes, int64_t W) {
+    if (check_common(dtype, B, L, d, depth) != PATHSIG_OK) return 0;
+    LevelPlan plan;
+    bool all_dense;
+    if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
+    const DenseChoice dc =
+        dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
+    return align_up((size_t)(B * (L - 1) * d) * elem_size(dtype)) + (dc.usable ? dc.backward_workspace : 0) + 256;
+}
+
+int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                         int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                         const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                         void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = check_common(dtype, B, L, d, depth);
+    if (rc != PATHSIG_OK) return rc;
+    if (B > 0 && (!path || !grad_path)) {
+        set_error("path and grad_path must not be NULL");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (windows && W < 0) {
+        set_error("W must be >= 0");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (dtype == PATHSIG_F32)
+        return sig_backward_t<float>(path, sig, grad_sig, grad_path, B, L, d, depth, level_sizes, encoded_words,
+                                     n_encoded, windows, W, workspace, workspace_bytes, (hipStream_t)stream);
+    return sig_backward_t<double>(path, sig, grad_sig, grad_path, B, L, d, depth, level_sizes, encoded_words,
+                                  n_encoded, windows, W, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, int64_t rows, int64_t d, int depth,
+                           int64_t top_size, const int64_t *top_words, void *stream) {
+    int rc = check_logsig(dtype, rows, d, depth, top_size);
+    if (rc != PATHSIG_OK) return rc;
+    if (rows == 0) return PATHSIG_OK;
+    if (!sig || !logsig || !P) {
+        set_error("sig, logsig and P must not be NULL");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (top_size != checked_pow(d, depth) && top_size > 0 && !top_words) {
+        set_error("top_words is NULL but the top level is not dense");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    hipError_t e;
+    if (dtype == PATHSIG_F32)
+        e = launch_logsig_forward<float>((const float *)sig, (float *)logsig, (float *)P, rows, d, depth, top_size,
+                                         top_words, (hipStream_t)stream);
+    else
+        e = launch_logsig_forward<double>((const double *)sig, (double *)logsig, (double *)P, rows, d, depth, top_size,
+                                          top_words, (hipStream_t)stream);
+    if (e != hipSuccess) return launch_failed(e, "logsig forward launch");
+    return PATHSIG_OK;
+}
+
+size_t pathsig_logsig_backward_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
+    if (check_logsig(dtype, rows, d, depth, top_size) != PATHSIG_OK) return 0;
+    return align_up((size_t)(rows * lower_columns(d, depth) * depth) * elem_size(dtype)) + 256;
+}
+
+int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_logsig, void *grad_sig, int dtype,
+                            int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
+                            void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = check_logsig(dtype, rows, d, depth, top_size);
+    if (rc != PATHSIG_OK) return rc;
+    if (rows == 0) return PATHSIG_OK;
+    if (!sig || !P || !grad_logsig || !grad_sig) {
+        set_error("sig, P, grad_logsig and grad_sig must not be NULL");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (top_size != checked_pow(d, depth) && top_size > 0 && !top_words) {
+        set_error("top_words is NULL but the top level is not dense");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    const size_t need = (size_t)(rows * lower_columns(d, depth) * depth) * elem_size(dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    hipError_t e;
+    if (dtype == PATHSIG_F32)
+        e = launch_logsig_backward<float>((const float *)sig, (const float *)P, (const float *)grad_logsig,
+                                          (float *)grad_sig, (float *)workspace, rows, d, depth, top_size, top_words,
+                                          (hipStream_t)stream);
+    else
+        e = launch_logsig_backward<double>((const double *)sig, (const double *)P, (const double *)grad_logsig,
+                                           (double *)grad_sig, (double *)workspace, rows, d, depth, top_size, top_words,
+                                           (hipStream_t)stream);
+    if (e != hipSuccess) return launch_failed(e, "logsig backward launch");
+    return PATHSIG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,396 @@
+// General signature kernels: one lane per requested word, any path dimension, any depth <= 12,
+// any word projection, any windows.  These are the kernels every call can fall back to; the
+// register-tiled dense kernels in dense_kernels.hip take over for the shapes they are built for.
+//
+// A lane that owns the word w = (w_1..w_n) carries the signature values of the prefixes of w
+// (a chain of n+1 numbers) and sweeps the window once.  Per increment it evaluates, for every
+// target level m = n..1, the Horner chain
+//     s_1 = 1/m,  tmp_j = p_j + s_j * dx[w_j],  s_{j+1} = tmp_j / (m - j),   p_m += s_m * dx[w_m]
+// which is S <- S (x) exp(dx) restricted to the chain (reference: src/pathsig/forward/sig_kernels.cu:129-154).
+// The backward lane carries the chain rolled back with exp(-dx) and the adjoint of the chain, and
+// back-propagates through the same Horner chains; this needs O(n^2) work per increment
+// (the reference assembles prefix x segment x suffix products in O(n^3),
+// src/pathsig/backward/sig_backward_kernels.cu:204-253).  Increments of a tile of time steps are
+// staged once per block in LDS; per-letter gradient sums are collected in LDS and flushed to the
+// per-increment accumulator with one atomic per (step, letter) per block.
+#include "common.hpp"
+
+namespace psig {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T>
+__device__ __forceinline__ T fma_t(T a, T b, T c);
+template <>
+__device__ __forceinline__ float fma_t<float>(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+template <>
+__device__ __forceinline__ double fma_t<double>(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ int find_level(const LevelPlan &plan, int64_t blk) {
+    int deg = 1;
+    while (deg < plan.depth && blk >= plan.block_begin[deg + 1]) ++deg;
+    return deg;
+}
+
+struct WindowSpan {
+    int64_t start, steps;
+};
+
+__device__ __forceinline__ WindowSpan window_span(const SigShape &shape, int64_t w) {
+    int64_t start = 0, end = shape.L;
+    if (shape.windows) {
+        start = shape.windows[2 * w];
+        end = shape.windows[2 * w + 1];
+        start = start < 0 ? 0 : (start > shape.L ? shape.L : start);
+        end = end < 0 ? 0 : (end > shape.L ? shape.L : end);
+    }
+    int64_t steps = end - start - 1;
+    return {start, steps < 0 ? 0 : steps};
+}
+
+template <int DEG>
+__device__ __forceinline__ void decode_letters(uint64_t code, uint64_t d, int (&l)[DEG]) {
+#pragma unroll
+    for (int pos = DEG - 1; pos >= 0; --pos) {
+        const uint64_t q = code / d;
+        l[pos] = (int)(code - q * d);
+        code = q;
+    }
+}
+
+// one forward Horner/Chen step on the chain p[0..TOP]; sign = +1 forward, -1 roll-back
+template <typename T, int DEG, int TOP>
+__device__ __forceinline__ void chain_step(T (&p)[DEG + 1], const T (&dl)[DEG], T sign) {
+#pragma unroll
+    for (int m = TOP; m >= 1; --m) {
+        T s = sign * Recip<T>::of(m);
+#pragma unroll
+        for (int j = 1; j < m; ++j) {
+            const T tmp = fma_t<T>(s, dl[j - 1], p[j]);
+            s = sign * tmp * Recip<T>::of(m - j);
+        }
+        p[m] = fma_t<T>(s, dl[m - 1], p[m]);
+    }
+}
+
+template <typename T, int DEG>
+__device__ void forward_body(const T *__restrict__ path, T *__restrict__ sig, const SigShape &shape,
+                             const LevelPlan &plan, const int64_t *__restrict__ codes, int64_t row, int64_t blk_in_level,
+                             int tile, T *sdx) {
+    const int tid = threadIdx.x;
+    const int64_t d = shape.d;
+    const int64_t word_idx = blk_in_level * kBlock + tid;
+    const bool active = word_idx < plan.size[DEG];
+    uint64_t code = 0;
+    if (active) code = plan.code_off[DEG] >= 0 ? (uint64_t)codes[plan.code_off[DEG] + word_idx] : (uint64_t)word_idx;
+    int l[DEG];
+    decode_letters<DEG>(code, (uint64_t)d, l);
+
+    const int64_t b = row / shape.W, w = row - b * shape.W;
+    const WindowSpan span = window_span(shape, w);
+    const T *x = path + (b * shape.L + span.start) * d;
+
+    T p[DEG + 1];
+    p[0] = T(1);
+#pragma unroll
+    for (int k = 1; k <= DEG; ++k) p[k] = T(0);
+
+    for (int64_t t0 = 0; t0 < span.steps; t0 += tile) {
+        const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
+        const T *xw = x + t0 * d;
+        __syncthreads();
+        for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) sdx[idx] = xw[idx + d] - xw[idx];
+        __syncthreads();
+        if (active) {
+            for (int tt = 0; tt < nt; ++tt) {
+                const T *dxr = sdx + (int64_t)tt * d;
+                T dl[DEG];
+#pragma unroll
+                for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
+                chain_step<T, DEG, DEG>(p, dl, T(1));
+            }
+        }
+    }
+    if (active) sig[row * plan.sig_size + plan.out_off[DEG] + word_idx] = p[DEG];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) words_forward_kernel(const T *__restrict__ path, T *__restrict__ sig,
+                                                               SigShape shape, LevelPlan plan,
+                                                               const int64_t *__restrict__ codes, int tile) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *sdx = reinterpret_cast<T *>(smem);
+    const int64_t per_row = plan.block_begin[plan.depth + 1];
+    const int64_t row = (int64_t)blockIdx.x / per_row;
+    const int64_t blk = (int64_t)blockIdx.x - row * per_row;
+    const int deg = find_level(plan, blk);
+    const int64_t bl = blk - plan.block_begin[deg];
+    switch (deg) {
+#define PSIG_CASE(N) \
+    case N: forward_body<T, N>(path, sig, shape, plan, codes, row, bl, tile, sdx); break;
+        PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
+        PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
+#undef PSIG_CASE
+        default: break;
+    }
+}
+
+template <typename T, int DEG>
+__device__ void backward_body(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
+                              T *__restrict__ grad_inc, const SigShape &shape, const LevelPlan &plan,
+                              const int64_t *__restrict__ codes, int64_t row, int64_t blk_in_level, int tile, T *sdx,
+                              T *sacc) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int64_t d = shape.d;
+    const int64_t word_idx = blk_in_level * kBlock + tid;
+    const bool active = word_idx < plan.size[DEG];
+    uint64_t code = 0;
+    if (active) code = plan.code_off[DEG] >= 0 ? (uint64_t)codes[plan.code_off[DEG] + word_idx] : (uint64_t)word_idx;
+    int l[DEG];
+    decode_letters<DEG>(code, (uint64_t)d, l);
+
+    // letter positions at which the whole wave holds the same letter are summed across the wave
+    // before they touch LDS
+    unsigned uniform_mask = 0;
+#pragma unroll
+    for (int k = 0; k < DEG; ++k) {
+        const int first = __shfl(l[k], 0, kWave);
+        if (__all(l[k] == first)) uniform_mask |= 1u << k;
+    }
+
+    const int64_t b = row / shape.W, w = row - b * shape.W;
+    const WindowSpan span = window_span(shape, w);
+    const T *x = path + (b * shape.L + span.start) * d;
+    T *ginc = grad_inc + (b * (shape.L - 1) + span.start) * d;
+    const T *srow = sig + row * plan.sig_size;
+
+    // chain of prefix values at the right end of the window (levels < DEG)
+    T p[DEG + 1];
+    p[0] = T(1);
+#pragma unroll
+    for (int k = 1; k <= DEG; ++k) p[k] = T(0);
+    if (plan.from_saved[DEG]) {
+        if (active) {
+            uint64_t off = 0, width = (uint64_t)d, pref = 0;
+#pragma unroll
+            for (int k = 1; k < DEG; ++k) {
+                pref = pref * (uint64_t)d + (uint64_t)l[k - 1];
+                p[k] = srow[off + pref];
+                off += width;
+                width *= (uint64_t)d;
+            }
+        }
+    } else if (DEG > 1) {
+        for (int64_t t0 = 0; t0 < span.steps; t0 += tile) {
+            const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
+            const T *xw = x + t0 * d;
+            __syncthreads();
+            for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) sdx[idx] = xw[idx + d] - xw[idx];
+            __syncthreads();
+            if (active) {
+                for (int tt = 0; tt < nt; ++tt) {
+                    const T *dxr = sdx + (int64_t)tt * d;
+                    T dl[DEG];
+#pragma unroll
+                    for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
+                    chain_step<T, DEG, DEG - 1>(p, dl, T(1));
+                }
+            }
+        }
+    }
+
+    // adjoint of the chain: h[k] = dL/dS(w_1..w_k) as far as this word contributes
+    T h[DEG + 1];
+#pragma unroll
+    for (int k = 0; k <= DEG; ++k) h[k] = T(0);
+    h[DEG] = active ? grad_sig[row * plan.sig_size + plan.out_off[DEG] + word_idx] : T(0);
+
+    const int64_t ntiles = (span.steps + tile - 1) / tile;
+    for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
+        const int64_t t0 = ti * tile;
+        const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
+        const T *xw = x + t0 * d;
+        __syncthreads();
+        for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) {
+            sdx[idx] = xw[idx + d] - xw[idx];
+            sacc[idx] = T(0);
+        }
+        __syncthreads();
+        if (active || uniform_mask) {
+            for (int tt = nt - 1; tt >= 0; --tt) {
+                const T *dxr = sdx + (int64_t)tt * d;
+                T *acc = sacc + (int64_t)tt * d;
+                T dl[DEG];
+#pragma unroll
+                for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
+                // S_t = S_{t+1} (x) exp(-dx_t) on the chain (levels < DEG are all the adjoint needs)
+                chain_step<T, DEG, DEG - 1>(p, dl, T(-1));
+                T gl[DEG];
+#pragma unroll
+                for (int k = 0; k < DEG; ++k) gl[k] = T(0);
+#pragma unroll
+                for (int m = 1; m <= DEG; ++m) {
+                    T s[DEG + 1];
+                    s[1] = Recip<T>::of(m);
+#pragma unroll
+                    for (int j = 1; j < m; ++j) {
+                        const T tmp = fma_t<T>(s[j], dl[j - 1], p[j]);
+                        s[j + 1] = tmp * Recip<T>::of(m - j);
+                    }
+                    T gt = h[m];
+#pragma unroll
+                    for (int j = m; j >= 1; --j) {
+                        gl[j - 1] = fma_t<T>(gt, s[j], gl[j - 1]);
+                        if (j > 1) {
+                            gt = gt * dl[j - 1] * Recip<T>::of(m - j + 1);
+                            h[j - 1] += gt;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < DEG; ++k) {
+                    if (uniform_mask & (1u << k)) {
+                        const T v = wave_sum<T>(gl[k]);
+                        if (lane == 0 && v != T(0)) atomicAdd(&acc[l[k]], v);
+                    } else if (gl[k] != T(0)) {
+                        atomicAdd(&acc[l[k]], gl[k]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) {
+            const T v = sacc[idx];
+            if (v != T(0)) atomicAdd(&ginc[t0 * d + idx], v);
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) words_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig,
+                                                                const T *__restrict__ grad_sig, T *__restrict__ grad_inc,
+                                                                SigShape shape, LevelPlan plan,
+                                                                const int64_t *__restrict__ codes, int tile) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *sdx = reinterpret_cast<T *>(smem);
+    T *sacc = sdx + (int64_t)tile * shape.d;
+    const int64_t per_row = plan.block_begin[plan.depth + 1];
+    const int64_t row = (int64_t)blockIdx.x / per_row;
+    const int64_t blk = (int64_t)blockIdx.x - row * per_row;
+    const int deg = find_level(plan, blk);
+    const int64_t bl = blk - plan.block_begin[deg];
+    switch (deg) {
+#define PSIG_CASE(N) \
+    case N: backward_body<T, N>(path, sig, grad_sig, grad_inc, shape, plan, codes, row, bl, tile, sdx, sacc); break;
+        PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
+        PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
+#undef PSIG_CASE
+        default: break;
+    }
+}
+
+template <typename T>
+__global__ void fill_zero_kernel(T *__restrict__ ptr, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) ptr[i] = T(0);
+}
+
+// dL/dx[t] = dL/d(dx[t-1]) - dL/d(dx[t]) with one-sided ends
+// (reference: src/pathsig/backward/sig_backward_kernels.cu:347-377; 64-bit indices here)
+template <typename T>
+__global__ void increments_to_path_kernel(const T *__restrict__ ginc, T *__restrict__ gpath, int64_t B, int64_t L,
+                                          int64_t d) {
+    const int64_t total = B * L * d;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t b = i / (L * d);
+        const int64_t rem = i - b * L * d;
+        const int64_t t = rem / d;
+        const int64_t a = rem - t * d;
+        const T *g = ginc + b * (L - 1) * d + a;
+        const T left = t > 0 ? g[(t - 1) * d] : T(0);
+        const T right = t < L - 1 ? g[t * d] : T(0);
+        gpath[i] = left - right;
+    }
+}
+
+int pick_tile(int64_t d, size_t elem, int64_t max_steps, int arrays) {
+    const int64_t budget = 16384 / arrays;
+    int64_t tile = budget / (int64_t)(d * elem);
+    if (tile < 1) tile = 1;
+    if (tile > 128) tile = 128;
+    if (tile > max_steps) tile = max_steps;
+    return (int)(tile < 1 ? 1 : tile);
+}
+
+}  // namespace
+
+template <typename T>
+hipError_t launch_words_forward(const T *path, T *sig, const SigShape &shape, const LevelPlan &plan,
+                                const int64_t *codes, hipStream_t stream) {
+    const int64_t per_row = plan.block_begin[plan.depth + 1];
+    const int64_t blocks = per_row * shape.B * shape.W;
+    if (blocks == 0) return hipSuccess;
+    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 1);
+    const size_t lds = (size_t)tile * shape.d * sizeof(T);
+    hipLaunchKernelGGL(words_forward_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), lds, stream, path, sig, shape,
+                       plan, codes, tile);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
+                                 const LevelPlan &plan, const int64_t *codes, hipStream_t stream) {
+    const int64_t per_row = plan.block_begin[plan.depth + 1];
+    const int64_t blocks = per_row * shape.B * shape.W;
+    if (blocks == 0) return hipSuccess;
+    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 2);
+    const size_t lds = (size_t)2 * tile * shape.d * sizeof(T);
+    hipLaunchKernelGGL(words_backward_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), lds, stream, path, sig,
+                       grad_sig, grad_inc, shape, plan, codes, tile);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream) {
+    if (n <= 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_zero_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, ptr, n);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
+                                     hipStream_t stream) {
+    const int64_t n = B * L * d;
+    if (n <= 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(increments_to_path_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_inc, grad_path,
+                       B, L, d);
+    return hipGetLastError();
+}
+
+#define PSIG_INSTANTIATE(T)                                                                                         \
+    template hipError_t launch_words_forward<T>(const T *, T *, const SigShape &, const LevelPlan &, const int64_t *, \
+                                                hipStream_t);                                                       \
+    template hipError_t launch_words_backward<T>(const T *, const T *, const T *, T *, const SigShape &,            \
+                                                 const LevelPlan &, const int64_t *, hipStream_t);                  \
+    template hipError_t launch_fill_zero<T>(T *, int64_t, hipStream_t);                                             \
+    template hipError_t launch_increments_to_path<T>(const T *, T *, int64_t, int64_t, int64_t, hipStream_t);
+PSIG_INSTANTIATE(float)
+PSIG_INSTANTIATE(double)
+#undef PSIG_INSTANTIATE
+
+}  // namespace psig

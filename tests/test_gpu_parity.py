@@ -1,0 +1,252 @@
+"""Parity of the HIP kernels (through the torch ops, i.e. through the C ABI) with the CPU checkers.
+
+Tolerances (max|got-want| / max(1, max|want|), the metric of the reference's `tests/test_sig.py:88-91`):
+fp64 1e-12, fp32 1e-5, as the build target states.  Index and layout checks are exact.
+"""
+from __future__ import annotations
+
+import pytest
+import torch
+
+from oracle import tensor_oracle as TO
+from tests.helpers import brownian_path, randn, random_word_set, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float64: 1e-12, torch.float32: 1e-5}
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ps():
+    import pathsig_amd
+    return pathsig_amd
+
+
+def _empty_i64():
+    return torch.empty(0, dtype=torch.int64, device=DEV)
+
+
+def _run_sig(ps, path_cpu, depth, dtype, projection=None, windows=None, G=None):
+    """Forward (+ backward when G is given) on the GPU; returns CPU tensors."""
+    x = path_cpu.to(dtype).to(DEV).requires_grad_(G is not None)
+    win = None if windows is None else torch.tensor(windows, dtype=torch.int64, device=DEV)
+    mod = ps.Signature(depth=depth, projection=projection, windows=win)
+    out = mod(x)
+    grad = None
+    if G is not None:
+        (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+        grad = grad.cpu()
+    return out.detach().cpu(), grad
+
+
+def _plan(projection):
+    if projection is None:
+        return None, None
+    return projection.level_sizes, projection._codes
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,L,B", [
+    (2, 1, 5, 3), (2, 2, 9, 2), (3, 3, 17, 4), (2, 6, 33, 3), (4, 4, 20, 5), (5, 3, 12, 2), (3, 5, 40, 2),
+    (7, 2, 6, 3), (2, 8, 11, 2), (2, 12, 6, 1), (33, 2, 7, 2), (4, 6, 24, 2), (6, 4, 2, 3),
+])
+def test_dense_forward_backward(ps, dtype, d, depth, L, B):
+    path = brownian_path(B, L, d, seed=100 + d * 13 + depth) * 3.0
+    want = TO.signature(path, depth)
+    G = randn(tuple(want.shape), seed=7)
+    got, grad = _run_sig(ps, path, depth, dtype, G=G)
+    assert got.shape == want.shape
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_windows(ps, dtype):
+    d, depth, L, B = 3, 4, 30, 3
+    path = brownian_path(B, L, d, seed=21) * 2.0
+    wins = [(0, 30), (3, 5), (2, 19), (15, 30), (4, 6), (10, 12), (0, 2), (28, 30), (5, 25), (5, 25)]
+    want = TO.compute_signature(path, depth, windows=wins)
+    G = randn(tuple(want.shape), seed=22)
+    got, grad = _run_sig(ps, path, depth, dtype, windows=wins, G=G)
+    assert got.shape == (B, len(wins), TO.dense_size(d, depth))
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth, windows=wins)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+def test_degenerate_windows_give_zero(ps):
+    d, depth = 2, 3
+    path = brownian_path(2, 10, d, seed=23)
+    wins = [(4, 5), (6, 6), (0, 10)]
+    got, grad = _run_sig(ps, path, depth, torch.float64, windows=wins,
+                         G=torch.ones(2, 3, TO.dense_size(d, depth), dtype=torch.float64))
+    assert got[:, 0].abs().max() == 0 and got[:, 1].abs().max() == 0
+    assert rel_err(got[:, 2], TO.signature(path, depth)) < 1e-12
+    assert torch.isfinite(grad).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("kind", ["words", "lyndon", "gap", "all_words", "full_levels"])
+def test_projections(ps, dtype, kind):
+    d, depth, L, B = 3, 4, 15, 3
+    if kind == "words":
+        proj = ps.projections.words(random_word_set(d, 1, 4, 40, seed=5), depth=depth, path_dim=d)
+    elif kind == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    elif kind == "gap":
+        proj = ps.projections.words([(1,), (0, 1, 2), (2, 2, 1), (1, 0, 0, 2), (1, 0, 0, 2)], depth=depth, path_dim=d)
+    elif kind == "all_words":
+        import itertools
+        words = [w for n in range(1, depth + 1) for w in itertools.product(range(d), repeat=n)]
+        proj = ps.projections.words(words, depth=depth, path_dim=d)
+        assert proj._codes == []
+    else:
+        proj = ps.projections.words(random_word_set(d, 3, 4, 20, seed=6), depth=depth, path_dim=d, full_levels=(1, 2))
+    sizes, codes = _plan(proj)
+    path = brownian_path(B, L, d, seed=31) * 2.0
+    want = TO.compute_signature(path, depth, sizes, codes)
+    G = randn(tuple(want.shape), seed=32)
+    got, grad = _run_sig(ps, path, depth, dtype, projection=proj, G=G)
+    assert got.shape == (B, proj.sig_size)
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth, sizes, codes)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+def test_projection_with_windows(ps):
+    d, depth, L, B = 4, 3, 20, 2
+    proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    wins = [(0, 10), (5, 20), (7, 9)]
+    path = brownian_path(B, L, d, seed=33)
+    sizes, codes = _plan(proj)
+    want = TO.compute_signature(path, depth, sizes, codes, wins)
+    G = randn(tuple(want.shape), seed=34)
+    got, grad = _run_sig(ps, path, depth, torch.float64, projection=proj, windows=wins, G=G)
+    assert rel_err(got, want) < 1e-12
+    assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes, wins)) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------
+# log-signature
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", [(2, 1), (2, 5), (3, 4), (4, 3), (5, 2)])
+def test_logsignature_dense(ps, dtype, d, depth):
+    B, L = 3, 14
+    path = brownian_path(B, L, d, seed=41) * 2.0
+    want = TO.logsignature(path, depth)
+    G = randn(tuple(want.shape), seed=42)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    out = ps.LogSignature(depth=depth)(x)
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    assert rel_err(out.detach(), want) < TOL[dtype]
+    xr = path.clone().requires_grad_(True)
+    (want_grad,) = torch.autograd.grad(TO.logsignature(xr, depth), xr, G)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,windows", [(3, 4, None), (2, 5, None), (4, 3, [(0, 9), (4, 14), (6, 8)])])
+def test_logsignature_lyndon(ps, dtype, d, depth, windows):
+    B, L = 3, 14
+    proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    path = brownian_path(B, L, d, seed=43) * 2.0
+    offs = TO.dense_level_offsets(d, depth)
+    cols = []
+    it = iter(proj._codes)
+    for k in range(1, depth + 1):
+        if proj.level_sizes[k] == d ** k:
+            cols += list(range(offs[k], offs[k + 1]))
+        else:
+            cols += [offs[k] + next(it) for _ in range(proj.level_sizes[k])]
+    cols = torch.tensor(cols)
+
+    def ref(x):
+        return TO.logsignature(x, depth, windows).index_select(-1, cols)
+
+    want = ref(path)
+    G = randn(tuple(want.shape), seed=44)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    win = None if windows is None else torch.tensor(windows, dtype=torch.int32, device=DEV)
+    out = ps.LogSignature(depth=depth, projection=proj, windows=win)(x)
+    assert out.shape == want.shape
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    assert rel_err(out.detach(), want) < TOL[dtype]
+    xr = path.clone().requires_grad_(True)
+    (want_grad,) = torch.autograd.grad(ref(xr), xr, G)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+def test_sig_to_logsig_cache_layout(ps):
+    """P[idx*depth + m-1] as the reference lays it out (`sig_kernels.cu:184,215-216`), every entry written."""
+    d, depth, B = 3, 4, 2
+    top = [5, 80, 17, 17, 2]
+    path = brownian_path(B, 9, d, seed=45)
+    dense = TO.signature(path, depth)
+    cols = TO.hybrid_columns(d, depth, len(top), top)
+    hyb = dense[:, cols]
+    want_log, want_P = TO.sig_to_logsig(hyb, depth, d, len(top), top)
+    sizes = [0] + [d ** k for k in range(1, depth)] + [len(top)]
+    words = torch.tensor(top, dtype=torch.int64, device=DEV)
+    logsig, P = torch.ops.pathsig.sig_to_logsig(hyb.to(DEV), depth, d, True, words, sizes)
+    assert P.shape == (B, len(cols) * depth)
+    assert rel_err(logsig, want_log) < 1e-12
+    assert rel_err(P, want_P) < 1e-12
+    g = randn(tuple(hyb.shape), seed=46)
+    got = torch.ops.pathsig.logsig_backward(hyb.to(DEV), P, g.to(DEV), depth, True, words, sizes)
+    assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------
+# behaviour at the operator boundary
+# ------------------------------------------------------------------------------------------------
+def test_errors(ps):
+    x = torch.zeros(2, 5, 3, device=DEV)
+    with pytest.raises(ValueError):
+        ps.Signature(depth=0)
+    with pytest.raises(ValueError):
+        ps.Signature(depth=13)
+    with pytest.raises(TypeError):
+        ps.Signature(depth=2, windows=torch.zeros(3, 2, dtype=torch.int64))
+    with pytest.raises(TypeError):
+        ps.Signature(depth=2, windows=torch.zeros(3, 3, dtype=torch.int64, device=DEV))
+    with pytest.raises(RuntimeError):
+        ps.Signature(depth=2)(torch.zeros(2, 1, 3, device=DEV))
+    with pytest.raises(RuntimeError):
+        ps.Signature(depth=2)(torch.zeros(2, 5, 3, device=DEV, dtype=torch.float16))
+    with pytest.raises(RuntimeError):
+        ps.Signature(depth=2)(torch.zeros(5, 3, device=DEV))
+    assert ps.Signature(depth=2)(x).shape == (2, 12)
+
+
+def test_non_contiguous_and_empty_batch(ps):
+    d, depth = 3, 3
+    base = brownian_path(2, 8, 2 * d, seed=51)
+    view = base.to(DEV)[:, :, ::2]
+    got = ps.Signature(depth=depth)(view)
+    assert rel_err(got, TO.signature(base[:, :, ::2].contiguous(), depth)) < 1e-12
+    empty = ps.Signature(depth=depth)(torch.zeros(0, 8, d, device=DEV, dtype=torch.float64))
+    assert empty.shape == (0, TO.dense_size(d, depth))
+
+
+def test_state_dict_buffers(ps):
+    proj = ps.projections.lyndon(depth=3, path_dim=3)
+    win = torch.tensor([[0, 4], [2, 6]], device=DEV)
+    sd = ps.Signature(depth=3, projection=proj, windows=win).state_dict()
+    assert set(sd) == {"_windows", "_encoded_words"} and sd["_windows"].dtype == torch.int32
+    assert ps.Signature(depth=3).state_dict() == {}
+    sd = ps.LogSignature(depth=3, projection=proj).state_dict()
+    assert set(sd) == {"_encoded_words", "_top_words", "_indices_from_sig"}
+    assert ps.LogSignature(depth=3).state_dict() == {}
+
+
+def test_gradcheck(ps):
+    torch.manual_seed(0)
+    x = torch.randn(2, 6, 2, dtype=torch.float64, device=DEV, requires_grad=True)
+    assert torch.autograd.gradcheck(ps.Signature(depth=3), (x,), atol=1e-5, rtol=1e-3)
+    assert torch.autograd.gradcheck(ps.LogSignature(depth=3), (x,), atol=1e-5, rtol=1e-3)
+    proj = ps.projections.lyndon(depth=3, path_dim=2)
+    win = torch.tensor([[0, 4], [2, 6], [1, 3]], device=DEV)
+    assert torch.autograd.gradcheck(ps.LogSignature(depth=3, projection=proj, windows=win), (x,), atol=1e-5, rtol=1e-3)
