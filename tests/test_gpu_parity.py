@@ -250,3 +250,35 @@ def test_gradcheck(ps):
     proj = ps.projections.lyndon(depth=3, path_dim=2)
     win = torch.tensor([[0, 4], [2, 6], [1, 3]], device=DEV)
     assert torch.autograd.gradcheck(ps.LogSignature(depth=3, projection=proj, windows=win), (x,), atol=1e-5, rtol=1e-3)
+
+
+# ------------------------------------------------------------------------------------------------
+# shapes served by the register-tiled dense kernels (forward, backward, windows, long paths)
+# ------------------------------------------------------------------------------------------------
+TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", TILED)
+def test_tiled_shapes(ps, dtype, d, depth):
+    B, L = 3, 150  # more than one LDS tile of increments, not a multiple of the tile
+    path = brownian_path(B, L, d, seed=200 + d + depth)
+    want = TO.signature(path, depth)
+    G = randn(tuple(want.shape), seed=61)
+    got, grad = _run_sig(ps, path, depth, dtype, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(grad, TO.signature_vjp(path, G, depth)) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", [(4, 6), (6, 5), (8, 4)])
+def test_tiled_shapes_with_windows(ps, dtype, d, depth):
+    B, L = 2, 100
+    path = brownian_path(B, L, d, seed=300 + d)
+    wins = [(0, 100), (0, 64), (32, 96), (64, 100), (10, 12), (50, 50), (3, 80), (3, 80)]
+    want = TO.compute_signature(path, depth, windows=wins)
+    G = randn(tuple(want.shape), seed=62)
+    got, grad = _run_sig(ps, path, depth, dtype, windows=wins, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth, windows=wins)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
