@@ -19,6 +19,7 @@
 // step (which yields H_{t-1} and dL/d(dx_t)), and keeps the top level of H equal to the upstream
 // gradient.  Adjoint values of the shared chain nodes stay lane-private partial sums (everything they
 // feed is linear in them), so the only cross-lane operation is the final sum of D numbers per step.
+#include <cstdlib>
 #include <type_traits>
 
 #include "dense.hpp"
@@ -199,15 +200,24 @@ __device__ __forceinline__ Span unit_span(const SigShape &shape, int64_t w) {
     return {start, steps < 0 ? 0 : steps};
 }
 
+// chunk c of `chunks` equal parts of a span: steps [begin, end)
+__device__ __forceinline__ void chunk_range(int64_t steps, int chunks, int c, int64_t &begin, int64_t &end) {
+    begin = steps * c / chunks;
+    end = steps * (c + 1) / chunks;
+}
+
 constexpr int kTile = 64;  // increments staged in LDS at a time
+
+constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2) : 1; }
 
 template <int D, int N, int P>
 struct Geometry {
     static constexpr int kLanes = ipow(D, P);
     static constexpr int kWaves = (kLanes + kWave - 1) / kWave;
     static constexpr int kBlock = kWaves * kWave;
-    static constexpr int kFwdSub = trie_size(D, N - P);      // sub-trie levels P+1..N
-    static constexpr int kASub = trie_size(D, N - 1 - P);    // levels P+1..N-1
+    static constexpr int kFwdSub = trie_size(D, N - P);    // sub-trie levels P+1..N
+    static constexpr int kASub = trie_size(D, N - 1 - P);  // levels P+1..N-1
+    static constexpr int kDumpRegs = P + kASub;            // chain + sub-trie below the top level
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
         int64_t o = 0, w = 1;
         for (int i = 1; i < k; ++i) {
@@ -217,6 +227,7 @@ struct Geometry {
         return o;
     }
     static constexpr int64_t kSigSize = level_off(N + 1);
+    static constexpr int64_t kLowSize = level_off(N);  // levels 1..N-1
 };
 
 // letters of the lane's prefix, most significant first
@@ -230,11 +241,161 @@ __device__ __forceinline__ void prefix_letters(int pu, int (&u)[P]) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// forward
+// lane state <-> dense layout in memory
+// ---------------------------------------------------------------------------------------------
+// Reads the chain a[1..P] and the sub-trie levels P+1..TOP of prefix pu from a dense-layout row.
+template <typename T, int D, int P, int TOP, int SUB>
+__device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bool active, T (&a)[P + 1], T (&sub)[SUB]) {
+    using G = Geometry<D, TOP, P>;
+    int rest = 1;
+#pragma unroll
+    for (int j = P; j >= 1; --j) {
+        a[j] = active ? row[G::level_off(j) + pu / rest] : T(0);
+        rest *= D;
+    }
+    static_for<1, TOP - P + 1>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        constexpr int width = ipow(D, k);
+        constexpr int off = trie_size(D, k - 1);
+        const T *src = row + G::level_off(P + k) + (int64_t)pu * width;
+#pragma unroll
+        for (int i = 0; i < width; ++i) sub[off + i] = active ? src[i] : T(0);
+    });
+}
+
+template <typename T, int D, int P, int TOP, int SUB>
+__device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T (&a)[P + 1], const T (&sub)[SUB]) {
+    using G = Geometry<D, TOP, P>;
+    // chain values are written by the lane whose remaining prefix letters are all zero
+    int rest = 1;
+#pragma unroll
+    for (int j = P; j >= 1; --j) {
+        if (pu % rest == 0) row[G::level_off(j) + pu / rest] = a[j];
+        rest *= D;
+    }
+    static_for<1, TOP - P + 1>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        constexpr int width = ipow(D, k);
+        constexpr int off = trie_size(D, k - 1);
+        T *dst = row + G::level_off(P + k) + (int64_t)pu * width;
+#pragma unroll
+        for (int i = 0; i < width; ++i) dst[i] = sub[off + i];
+    });
+}
+
+// codes of the sub-words u_{k+1..i} of the lane's prefix, 0 <= k < i <= P
+template <int D, int P>
+struct SubWords {
+    int code[P + 1][P + 1];
+    __device__ __forceinline__ explicit SubWords(const int (&u)[P]) {
+#pragma unroll
+        for (int k = 0; k <= P; ++k) {
+            int c = 0;
+#pragma unroll
+            for (int i = 0; i <= P; ++i) {
+                if (i > k) c = c * D + u[i - 1];
+                code[k][i] = c;
+            }
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// A <- A (x) B on a lane's state (chain + sub-trie levels P+1..TOP); B is a dense-layout row.
+//   (A (x) B)(u v) = sum_{k<=P} A(u_1..u_k) B(u_{k+1}..u_P v) + sum_{j<|v|} A(u v_1..v_j) B(v_{j+1}..) + A(u v)
+// Sub-trie levels go top-down and the chain last, so everything read is still the old A.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D, int P, int TOP, int SUB>
+__device__ __forceinline__ void apply_right(T (&a)[P + 1], T (&sub)[SUB], const T *__restrict__ B,
+                                            const SubWords<D, P> &sw) {
+    using G = Geometry<D, TOP, P>;
+    a[0] = T(1);
+    static_for<0, TOP - P>([&](auto rc) {
+        constexpr int r = TOP - P - decltype(rc)::value;  // TOP-P .. 1
+        constexpr int width = ipow(D, r);
+        constexpr int off = trie_size(D, r - 1);
+        T acc[width];
+#pragma unroll
+        for (int iv = 0; iv < width; ++iv) acc[iv] = sub[off + iv];
+        // own sub-trie values times the low words of B
+        static_for<1, r>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            constexpr int tail = ipow(D, r - j);
+            constexpr int offj = trie_size(D, j - 1);
+#pragma unroll
+            for (int iv = 0; iv < width; ++iv)
+                acc[iv] = fmad<T>(sub[offj + iv / tail], B[G::level_off(r - j) + iv % tail], acc[iv]);
+        });
+        // chain values times B at (suffix of the prefix) . v
+        static_for<0, P + 1>([&](auto kc) {
+            constexpr int k = decltype(kc)::value;
+            const T *run = B + G::level_off(P - k + r) + (int64_t)sw.code[k][P] * width;
+#pragma unroll
+            for (int iv = 0; iv < width; ++iv) acc[iv] = fmad<T>(a[k], run[iv], acc[iv]);
+        });
+#pragma unroll
+        for (int iv = 0; iv < width; ++iv) sub[off + iv] = acc[iv];
+    });
+#pragma unroll
+    for (int i = P; i >= 1; --i) {
+        T acc = a[i];
+#pragma unroll
+        for (int k = 0; k < i; ++k) acc = fmad<T>(a[k], B[G::level_off(i - k) + sw.code[k][i]], acc);
+        a[i] = acc;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// H <- H contracted on the right with B:  H'(w) = sum_s H(w s) B(s),  B(empty) = 1.
+// State: lane-private chain partials hc[1..P], sub-trie levels P+1..N (the top level never changes).
+// B is a dense-layout row with levels 1..N-1.  The chain goes first (ascending), then the sub-trie
+// levels top-down in depth, so everything read is still the old H.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D, int N, int P, int HSUB>
+__device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], const T *__restrict__ B,
+                                               const SubWords<D, P> &sw) {
+    using G = Geometry<D, N, P>;
+    constexpr int R = N - P;
+#pragma unroll
+    for (int i = 1; i <= P; ++i) {
+        T acc = hc[i];
+#pragma unroll
+        for (int i2 = i + 1; i2 <= P; ++i2) acc = fmad<T>(hc[i2], B[G::level_off(i2 - i) + sw.code[i][i2]], acc);
+        static_for<1, R + 1>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            constexpr int width = ipow(D, r);
+            constexpr int off = trie_size(D, r - 1);
+            const T *run = B + G::level_off(P - i + r) + (int64_t)sw.code[i][P] * width;
+#pragma unroll
+            for (int iv = 0; iv < width; ++iv) acc = fmad<T>(hsub[off + iv], run[iv], acc);
+        });
+        hc[i] = acc;
+    }
+    static_for<1, R>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;  // 1 .. R-1
+        constexpr int width = ipow(D, r);
+        constexpr int off = trie_size(D, r - 1);
+        static_for<1, R - r + 1>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;  // extension length
+            constexpr int ext = ipow(D, q);
+            constexpr int offq = trie_size(D, r + q - 1);
+#pragma unroll
+            for (int iv = 0; iv < width; ++iv) {
+                T acc = hsub[off + iv];
+#pragma unroll
+                for (int e = 0; e < ext; ++e) acc = fmad<T>(hsub[offq + iv * ext + e], B[G::level_off(q) + e], acc);
+                hsub[off + iv] = acc;
+            }
+        });
+    });
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward: one block per unit (row, chunk); writes the unit's signature as a dense-layout row
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, int N, int P>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
-    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ sig, SigShape shape) {
+    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
     __shared__ T sdx[kTile * D];
     const int pu = threadIdx.x;
@@ -242,9 +403,13 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
 
-    const int64_t row = blockIdx.x;
+    const int64_t unit = blockIdx.x;
+    const int64_t row = unit / chunks;
+    const int c = (int)(unit - row * chunks);
     const int64_t b = row / shape.W, w = row - b * shape.W;
     const Span span = unit_span(shape, w);
+    int64_t begin, end;
+    chunk_range(span.steps, chunks, c, begin, end);
     const T *x = path + (b * shape.L + span.start) * D;
 
     T a[P + 1];
@@ -254,8 +419,8 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 #pragma unroll
     for (int i = 0; i < G::kFwdSub; ++i) sub[i] = T(0);
 
-    for (int64_t t0 = 0; t0 < span.steps; t0 += kTile) {
-        const int nt = (int)((span.steps - t0) < kTile ? (span.steps - t0) : kTile);
+    for (int64_t t0 = begin; t0 < end; t0 += kTile) {
+        const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
         const T *xw = x + t0 * D;
         __syncthreads();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
@@ -269,35 +434,112 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
             StepTargets<T, D, P, N, false>::template run<G::kFwdSub>(a, sub, dx, dxp);
         }
     }
+    if (active) store_state<T, D, P, N, G::kFwdSub>(out + unit * G::kSigSize, pu, a, sub);
+}
 
-    if (!active) return;
-    T *out = sig + row * G::kSigSize;
-    // chain values are written by the lane whose remaining prefix letters are all zero
-    {
-        int rest = 1;  // D^(P-j)
-#pragma unroll
-        for (int j = P; j >= 1; --j) {
-            if (pu % rest == 0) out[G::level_off(j) + pu / rest] = a[j];
-            rest *= D;
-        }
-    }
-    static_for<1, N - P + 1>([&](auto kc) {
-        constexpr int k = decltype(kc)::value;
-        constexpr int width = ipow(D, k);
-        constexpr int off = trie_size(D, k - 1);
-        T *dst = out + G::level_off(P + k) + (int64_t)pu * width;
-#pragma unroll
-        for (int i = 0; i < width; ++i) dst[i] = sub[off + i];
-    });
+// product of the chunk signatures of one row, left to right
+template <typename T, int D, int N, int P>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+    dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks) {
+    using G = Geometry<D, N, P>;
+    const int pu = threadIdx.x;
+    const bool active = pu < G::kLanes;
+    int u[P];
+    prefix_letters<D, P>(active ? pu : 0, u);
+    const SubWords<D, P> sw(u);
+    const int64_t row = blockIdx.x;
+    const T *rows = chunk_sig + row * chunks * G::kSigSize;
+    T a[P + 1];
+    T sub[G::kFwdSub];
+    load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
+    for (int c = 1; c < chunks; ++c) apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
+    if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
 }
 
 // ---------------------------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int N, int P, bool ACCUMULATE>
+// Register dump of a lane's chain + sub-trie below the top level: element (reg, lane) of unit at
+// ((unit * kDumpRegs) + reg) * kBlock + lane.
+template <typename T, int D, int N, int P, int SUBN>
+__device__ __forceinline__ void dump_state(T *__restrict__ dst, int64_t unit, int lane, const T (&c)[P + 1],
+                                           const T (&sub)[SUBN]) {
+    using G = Geometry<D, N, P>;
+    T *base = dst + unit * G::kDumpRegs * G::kBlock + lane;
+#pragma unroll
+    for (int j = 1; j <= P; ++j) base[(j - 1) * G::kBlock] = c[j];
+#pragma unroll
+    for (int i = 0; i < G::kASub; ++i) base[(P + i) * G::kBlock] = sub[i];
+}
+
+template <typename T, int D, int N, int P, int SUBN>
+__device__ __forceinline__ void undump_state(const T *__restrict__ src, int64_t unit, int lane, T (&c)[P + 1],
+                                             T (&sub)[SUBN]) {
+    using G = Geometry<D, N, P>;
+    const T *base = src + unit * G::kDumpRegs * G::kBlock + lane;
+#pragma unroll
+    for (int j = 1; j <= P; ++j) c[j] = base[(j - 1) * G::kBlock];
+#pragma unroll
+    for (int i = 0; i < G::kASub; ++i) sub[i] = base[(P + i) * G::kBlock];
+}
+
+// initial adjoint state of a row: chain entries are lane-private partial sums, so only the lane whose
+// remaining prefix letters are zero starts from the upstream gradient
+template <typename T, int D, int N, int P>
+__device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu, bool active, T (&hc)[P + 1],
+                                             T (&hsub)[Geometry<D, N, P>::kFwdSub]) {
+    using G = Geometry<D, N, P>;
+    load_state<T, D, P, N, G::kFwdSub>(grow, pu, active, hc, hsub);
+    int rest = 1;
+#pragma unroll
+    for (int j = P; j >= 1; --j) {
+        if (pu % rest != 0) hc[j] = T(0);
+        rest *= D;
+    }
+    hc[0] = T(0);
+}
+
+// Per row: state at the right edge of every chunk.  blockIdx.y == 0: A_c = S_0 (x) .. (x) S_c (levels < N),
+// blockIdx.y == 1: H_c = adjoint of the signature at the right edge of chunk c.
+template <typename T, int D, int N, int P>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+    dense_scan_kernel(const T *__restrict__ chunk_low, const T *__restrict__ grad_sig, T *__restrict__ dumpA,
+                      T *__restrict__ dumpH, int chunks) {
+    using G = Geometry<D, N, P>;
+    constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
+    const int pu = threadIdx.x;
+    const bool active = pu < G::kLanes;
+    int u[P];
+    prefix_letters<D, P>(active ? pu : 0, u);
+    const SubWords<D, P> sw(u);
+    const int64_t row = blockIdx.x;
+    const T *rows = chunk_low + row * chunks * G::kLowSize;
+    if (blockIdx.y == 0) {
+        T a[P + 1];
+        T asub[kAS];
+        load_state<T, D, P, N - 1, kAS>(rows, pu, active, a, asub);
+        dump_state<T, D, N, P, kAS>(dumpA, row * chunks, pu, a, asub);
+        for (int c = 1; c < chunks; ++c) {
+            apply_right<T, D, P, N - 1, kAS>(a, asub, rows + (int64_t)c * G::kLowSize, sw);
+            dump_state<T, D, N, P, kAS>(dumpA, row * chunks + c, pu, a, asub);
+        }
+    } else {
+        T hc[P + 1];
+        T hsub[G::kFwdSub];
+        load_adjoint<T, D, N, P>(grad_sig + row * G::kSigSize, pu, active, hc, hsub);
+        dump_state<T, D, N, P, G::kFwdSub>(dumpH, row * chunks + chunks - 1, pu, hc, hsub);
+        for (int c = chunks - 1; c >= 1; --c) {
+            contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, rows + (int64_t)c * G::kLowSize, sw);
+            dump_state<T, D, N, P, G::kFwdSub>(dumpH, row * chunks + c - 1, pu, hc, hsub);
+        }
+    }
+}
+
+template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
-                          T *__restrict__ grad_inc, SigShape shape) {
+                          const T *__restrict__ dumpA, const T *__restrict__ dumpH, T *__restrict__ grad_inc,
+                          SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
     __shared__ T sdx[kTile * D];
     __shared__ T sg[G::kWaves][kTile * D];
@@ -308,48 +550,36 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
 
-    const int64_t row = blockIdx.x;
+    const int64_t unit = blockIdx.x;
+    const int64_t row = unit / chunks;
+    const int c = (int)(unit - row * chunks);
     const int64_t b = row / shape.W, w = row - b * shape.W;
     const Span span = unit_span(shape, w);
+    int64_t begin, end;
+    chunk_range(span.steps, chunks, c, begin, end);
     const T *x = path + (b * shape.L + span.start) * D;
     T *ginc = grad_inc + (b * (shape.L - 1) + span.start) * D;
-    const T *srow = sig + row * G::kSigSize;
     const T *grow = grad_sig + row * G::kSigSize;
 
-    // A: signature at the right end (levels < N).  H: upstream gradient; chain entries are lane-private
-    // partial sums, so only the lane whose remaining prefix letters are zero starts from the gradient.
-    T a[P + 1], hc[P + 1];
+    // A: signature at the right edge of the unit (levels < N).  H: adjoint at the right edge.
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
+    T a[P + 1], hc[P + 1];
     T asub[kAS];
     T hsub[G::kFwdSub];
-    a[0] = T(1);
-    hc[0] = T(0);
-    {
-        int rest = 1;
-#pragma unroll
-        for (int j = P; j >= 1; --j) {
-            const int64_t col = G::level_off(j) + pu / rest;
-            a[j] = (active && j < N) ? srow[col] : T(0);
-            hc[j] = (active && pu % rest == 0) ? grow[col] : T(0);
-            rest *= D;
-        }
+    load_adjoint<T, D, N, P>(grow, pu, active, hc, hsub);
+    if constexpr (CHUNKED) {
+        undump_state<T, D, N, P, kAS>(dumpA, unit, pu, a, asub);
+        undump_state<T, D, N, P, G::kFwdSub>(dumpH, unit, pu, hc, hsub);
+    } else {
+        load_state<T, D, P, N - 1, kAS>(sig + row * G::kSigSize, pu, active, a, asub);
     }
-    static_for<1, N - P + 1>([&](auto kc) {
-        constexpr int k = decltype(kc)::value;
-        constexpr int width = ipow(D, k);
-        constexpr int off = trie_size(D, k - 1);
-        const int64_t col = G::level_off(P + k) + (int64_t)pu * width;
-#pragma unroll
-        for (int i = 0; i < width; ++i) {
-            hsub[off + i] = active ? grow[col + i] : T(0);
-            if constexpr (k < N - P) asub[off + i] = active ? srow[col + i] : T(0);
-        }
-    });
+    a[0] = T(1);
 
-    const int64_t ntiles = (span.steps + kTile - 1) / kTile;
+    const int64_t len = end - begin;
+    const int64_t ntiles = (len + kTile - 1) / kTile;
     for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
-        const int64_t t0 = ti * kTile;
-        const int nt = (int)((span.steps - t0) < kTile ? (span.steps - t0) : kTile);
+        const int64_t t0 = begin + ti * kTile;
+        const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
         const T *xw = x + t0 * D;
         __syncthreads();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
@@ -368,7 +598,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 #pragma unroll
             for (int j = 0; j < P; ++j) gpre[j] = T(0);
             AdjTargets<T, D, N, P, 1>::template run<kAS, G::kFwdSub>(a, asub, hc, hsub, dx, dxp, gdx, gpre);
-            // letter a collects the sub-trie sums and the chain positions whose letter is a
+            // letter k collects the sub-trie sums and the chain positions whose letter is k
 #pragma unroll
             for (int k = 0; k < D; ++k) {
                 T v = gdx[k];
@@ -392,83 +622,169 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     }
 }
 
-// table of compiled shapes
-struct Variant {
-    int d, depth;
+// ---------------------------------------------------------------------------------------------
+// host side: table of compiled shapes and launch sequences
+// ---------------------------------------------------------------------------------------------
+// X(index, D, N, P): signature over D letters to depth N with lanes on prefixes of length P.  The
+// backward also runs the forward kernel of depth N-1 (same P) to get chunk signatures below the top level.
+#define PSIG_VARIANTS(X) X(0, 4, 6, 3) X(1, 8, 4, 2) X(2, 6, 5, 3) X(3, 4, 4, 2) X(4, 3, 5, 3) X(5, 2, 8, 5)
+
+struct VariantInfo {
+    int d, depth, block, dump_regs;
+    int64_t sig_size, low_size;
 };
-constexpr Variant kVariants[] = {{4, 6}, {8, 4}, {6, 5}, {4, 4}, {3, 5}, {2, 8}};
+
+template <int D, int N, int P>
+constexpr VariantInfo variant_info() {
+    using G = Geometry<D, N, P>;
+    return VariantInfo{D, N, G::kBlock, G::kDumpRegs, G::kSigSize, G::kLowSize};
+}
+
+#define PSIG_INFO(I, D, N, P) variant_info<D, N, P>(),
+constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
+#undef PSIG_INFO
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
+size_t pad256(size_t n) { return (n + 255) / 256 * 256; }
+
+// number of time chunks per row: enough waves to give every SIMD of the GPU about two, but chunks
+// of at least 16 increments
+int pick_chunks(int64_t rows, int block, int64_t L) {
+    const int64_t waves_per_row = block / kWave;
+    const int64_t want_waves = 2048;
+    int64_t c = (want_waves + rows * waves_per_row - 1) / (rows * waves_per_row);
+    const int64_t max_c = (L - 1) / 16;
+    if (c > max_c) c = max_c;
+    if (c > 64) c = 64;
+    if (c < 1) c = 1;
+    return (int)c;
+}
+
 template <typename T, int D, int N, int P>
-hipError_t run_forward(const T *path, T *sig, const SigShape &shape, hipStream_t stream) {
+hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
     const int64_t rows = shape.B * shape.W;
-    hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream, path, sig,
-                       shape);
+    if (chunks <= 1) {
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream, path,
+                           sig, shape, 1);
+        return hipGetLastError();
+    }
+    T *chunk_sig = (T *)workspace;
+    hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0, stream,
+                       path, chunk_sig, shape, chunks);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((dense_combine_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
+                       (const T *)chunk_sig, sig, chunks);
     return hipGetLastError();
 }
 
 template <typename T, int D, int N, int P>
-hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                        hipStream_t stream) {
+hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape, int chunks,
+                        void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
     const int64_t rows = shape.B * shape.W;
-    if (shape.windows) {
-        hipError_t e = launch_fill_zero<T>(grad_inc, shape.B * (shape.L - 1) * shape.d, stream);
+    const bool accumulate = shape.windows != nullptr;
+    hipError_t e;
+    if (accumulate) {
+        e = launch_fill_zero<T>(grad_inc, shape.B * (shape.L - 1) * shape.d, stream);
         if (e != hipSuccess) return e;
-        if (rows == 0) return hipSuccess;
-        hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
-                           path, sig, grad_sig, grad_inc, shape);
-    } else {
-        hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
-                           path, sig, grad_sig, grad_inc, shape);
     }
-    return hipGetLastError();
+    if (rows == 0) return hipSuccess;
+    if (chunks <= 1) {
+        if (accumulate)
+            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, false>), dim3((unsigned)rows), dim3(G::kBlock),
+                               0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr, grad_inc, shape,
+                               1);
+        else
+            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, false>), dim3((unsigned)rows),
+                               dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr,
+                               grad_inc, shape, 1);
+        return hipGetLastError();
+    }
+    if constexpr (N < 2) {
+        return hipErrorNotSupported;
+    } else {
+        const int64_t units = rows * chunks;
+        unsigned char *ws = (unsigned char *)workspace;
+        T *chunk_low = (T *)ws;
+        ws += pad256((size_t)units * G::kLowSize * sizeof(T));
+        T *dumpA = (T *)ws;
+        ws += pad256((size_t)units * G::kDumpRegs * G::kBlock * sizeof(T));
+        T *dumpH = (T *)ws;
+        // chunk signatures below the top level: the depth N-1 forward kernel on the same units
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P>), dim3((unsigned)units),
+                           dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((dense_scan_kernel<T, D, N, P>), dim3((unsigned)rows, 2), dim3(G::kBlock), 0, stream,
+                           (const T *)chunk_low, grad_sig, dumpA, dumpH, chunks);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        if (accumulate)
+            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units), dim3(G::kBlock),
+                               0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH, grad_inc, shape,
+                               chunks);
+        else
+            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
+                               dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
+                               grad_inc, shape, chunks);
+        return hipGetLastError();
+    }
 }
 
 }  // namespace
 
-DenseChoice dense_choice(size_t, int64_t d, int depth, bool all_dense, const int64_t *, int64_t B, int64_t, int64_t W,
-                         bool) {
+DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *, int64_t B, int64_t L,
+                         int64_t W, bool) {
     DenseChoice dc{false, -1, 1, 0, 0};
-    if (!all_dense) return dc;
-    if (B * W >= (int64_t(1) << 31)) return dc;
+    if (!all_dense || B <= 0 || W <= 0) return dc;
     for (int i = 0; i < kNumVariants; ++i) {
-        if (kVariants[i].d == d && kVariants[i].depth == depth) {
-            dc.usable = true;
-            dc.variant = i;
-            return dc;
+        const VariantInfo &v = kVariants[i];
+        if (v.d != d || v.depth != depth) continue;
+        const int64_t rows = B * W;
+        int chunks = pick_chunks(rows, v.block, L);
+        if (const char *env = getenv("PATHSIG_CHUNKS")) {
+            const int forced = atoi(env);
+            if (forced >= 1 && forced <= 1024) chunks = forced;
         }
+        if (rows * chunks >= (int64_t(1) << 31)) return dc;
+        dc.usable = true;
+        dc.variant = i;
+        dc.chunks = chunks;
+        if (chunks > 1) {
+            const size_t units = (size_t)rows * chunks;
+            dc.forward_workspace = pad256(units * v.sig_size * elem);
+            dc.backward_workspace = pad256(units * v.low_size * elem) +
+                                    2 * pad256(units * (size_t)v.dump_regs * v.block * elem);
+        }
+        return dc;
     }
     return dc;
 }
 
-#define PSIG_DISPATCH(CALL)                      \
-    switch (dc.variant) {                        \
-        case 0: return CALL(4, 6, 3);            \
-        case 1: return CALL(8, 4, 2);            \
-        case 2: return CALL(6, 5, 3);            \
-        case 3: return CALL(4, 4, 2);            \
-        case 4: return CALL(3, 5, 3);            \
-        case 5: return CALL(2, 8, 5);            \
-        default: return hipErrorNotSupported;    \
-    }
+#define PSIG_CASE_FWD(I, D, N, P) \
+    case I: return run_forward<T, D, N, P>(path, sig, shape, dc.chunks, workspace, stream);
+#define PSIG_CASE_BWD(I, D, N, P) \
+    case I: return run_backward<T, D, N, P>(path, sig, grad_sig, grad_inc, shape, dc.chunks, workspace, stream);
 
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const LevelPlan &, const int64_t *,
-                                const DenseChoice &dc, void *, hipStream_t stream) {
-#define PSIG_FWD(D, N, P) run_forward<T, D, N, P>(path, sig, shape, stream)
-    PSIG_DISPATCH(PSIG_FWD)
-#undef PSIG_FWD
+                                const DenseChoice &dc, void *workspace, hipStream_t stream) {
+    switch (dc.variant) {
+        PSIG_VARIANTS(PSIG_CASE_FWD)
+        default: return hipErrorNotSupported;
+    }
 }
 
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const LevelPlan &, const int64_t *, const DenseChoice &dc, void *,
+                                 const LevelPlan &, const int64_t *, const DenseChoice &dc, void *workspace,
                                  hipStream_t stream) {
-#define PSIG_BWD(D, N, P) run_backward<T, D, N, P>(path, sig, grad_sig, grad_inc, shape, stream)
-    PSIG_DISPATCH(PSIG_BWD)
-#undef PSIG_BWD
+    switch (dc.variant) {
+        PSIG_VARIANTS(PSIG_CASE_BWD)
+        default: return hipErrorNotSupported;
+    }
 }
 
 #define PSIG_INSTANTIATE(T)                                                                                  \

@@ -282,3 +282,32 @@ def test_tiled_shapes_with_windows(ps, dtype, d, depth):
     assert rel_err(got, want) < TOL[dtype]
     want_grad = TO.signature_vjp(path, G, depth, windows=wins)
     assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("chunks", ["2", "5", "16"])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", TILED)
+def test_tiled_shapes_time_chunked(ps, monkeypatch, chunks, dtype, d, depth):
+    """Long paths are cut into time chunks whose signatures are multiplied back together (Chen);
+    PATHSIG_CHUNKS forces the chunk count so that small inputs exercise that path too."""
+    monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
+    B, L = 2, 150
+    path = brownian_path(B, L, d, seed=400 + d + depth)
+    want = TO.signature(path, depth)
+    G = randn(tuple(want.shape), seed=63)
+    got, grad = _run_sig(ps, path, depth, dtype, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(grad, TO.signature_vjp(path, G, depth)) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("d,depth", [(4, 6), (6, 5)])
+def test_tiled_shapes_time_chunked_windows(ps, monkeypatch, d, depth):
+    monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+    B, L = 2, 100
+    path = brownian_path(B, L, d, seed=500 + d)
+    wins = [(0, 100), (0, 64), (32, 96), (64, 100), (10, 12), (50, 50), (3, 80), (97, 100)]  # some shorter than the chunk count
+    want = TO.compute_signature(path, depth, windows=wins)
+    G = randn(tuple(want.shape), seed=64)
+    got, grad = _run_sig(ps, path, depth, torch.float64, windows=wins, G=G)
+    assert rel_err(got, want) < 1e-12
+    assert rel_err(grad, TO.signature_vjp(path, G, depth, windows=wins)) < 1e-12
