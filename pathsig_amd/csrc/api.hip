@@ -141,8 +141,15 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
             set_error("workspace too small: need %zu bytes, got %zu", dc.forward_workspace, workspace_bytes);
             return PATHSIG_ERR_WORKSPACE;
         }
-        hipError_t e = launch_dense_forward<T>((const T *)path, (T *)sig, shape, plan, codes, dc, workspace, stream);
+        // a dense call writes straight into sig; an embedded projection goes through a dense buffer
+        T *dense = dc.embed ? (T *)workspace : (T *)sig;
+        void *rest = (unsigned char *)workspace + dc.dense_bytes;
+        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, rest, stream);
         if (e != hipSuccess) return launch_failed(e, "dense forward launch");
+        if (dc.embed) {
+            e = launch_gather_columns<T>(dense, (T *)sig, plan, d, codes, B * shape.W, stream);
+            if (e != hipSuccess) return launch_failed(e, "gather launch");
+        }
         return PATHSIG_OK;
     }
     hipError_t e = launch_words_forward<T>((const T *)path, (T *)sig, shape, plan, codes, stream);
@@ -172,9 +179,20 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     T *ginc = (T *)workspace;
     hipError_t e;
     if (dc.usable) {
-        void *extra = (unsigned char *)workspace + inc_bytes;
-        e = launch_dense_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan, codes, dc,
-                                     extra, stream);
+        unsigned char *extra = (unsigned char *)workspace + inc_bytes;
+        const T *gdense = (const T *)grad_sig;
+        if (dc.embed) {
+            // upstream gradient scattered into a zeroed dense buffer; the dense signature itself is not
+            // needed because the time-chunked backward rebuilds what it reads
+            T *buf = (T *)extra;
+            e = launch_fill_zero<T>(buf, (int64_t)(dc.dense_bytes / sizeof(T)), stream);
+            if (e != hipSuccess) return launch_failed(e, "fill launch");
+            e = launch_scatter_columns<T>((const T *)grad_sig, buf, plan, d, codes, B * shape.W, stream);
+            if (e != hipSuccess) return launch_failed(e, "scatter launch");
+            gdense = buf;
+        }
+        e = launch_dense_backward<T>((const T *)path, dc.embed ? (const T *)nullptr : (const T *)sig, gdense, ginc,
+                                     shape, dc, extra + dc.dense_bytes, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
     } else {
         e = launch_fill_zero<T>(ginc, B * (L - 1) * d, stream);

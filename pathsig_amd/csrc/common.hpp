@@ -34,6 +34,32 @@ struct SigShape {
 
 void set_error(const char *fmt, ...);
 
+#if defined(__HIPCC__)
+// Wave-wide sum of one value per lane; the total is valid in lane 63 only.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add_c(float v) {
+    // lanes outside ROW_MASK, and lanes whose source lane is invalid, add zero
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+__device__ __forceinline__ float wave_total(float v) {
+    v = dpp_add_c<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add_c<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add_c<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add_c<0x140, 0xF>(v);  // row_mirror: every lane now holds the sum of its row of 16
+    v = dpp_add_c<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add_c<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ double wave_total(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+#endif
+
 template <typename T>
 struct Recip {
     // 1/k for k = 1..12 as compile-time constants of type T
@@ -49,6 +75,13 @@ hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig,
                                  const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream);
+// projected layout <- dense layout (gather) and dense layout += projected layout (scatter; dense zeroed before)
+template <typename T>
+hipError_t launch_gather_columns(const T *dense, T *out, const LevelPlan &plan, int64_t d, const int64_t *codes,
+                                 int64_t rows, hipStream_t stream);
+template <typename T>
+hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan, int64_t d, const int64_t *codes,
+                                  int64_t rows, hipStream_t stream);
 template <typename T>
 hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
                                      hipStream_t stream);

@@ -7,21 +7,24 @@ namespace psig {
 
 struct DenseChoice {
     bool usable;                // a register-tiled kernel exists for this call
+    bool embed;                 // the call is a word projection that is computed densely and then gathered
     int variant;                // index into the table of compiled shapes
-    int chunks;                 // time chunks per (path, window)
-    size_t forward_workspace;   // bytes of scratch the forward needs
+    int fwd_chunks;             // time chunks per (path, window) in the forward
+    int bwd_chunks;             // ... and in the backward (at least 2 when embedding: no dense signature is saved)
+    size_t dense_bytes;         // embed: bytes of one dense [rows, S] buffer
+    size_t forward_workspace;   // bytes of scratch the forward needs (including the dense buffer)
     size_t backward_workspace;  // bytes of scratch the backward needs beyond the increment accumulator
 };
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,
                          int64_t L, int64_t W, bool windowed);
 
+// `sig` / `grad_sig` are dense-layout rows; `workspace` is the part of the scratch after any dense buffer.
 template <typename T>
-hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const LevelPlan &plan,
-                                const int64_t *codes, const DenseChoice &dc, void *workspace, hipStream_t stream);
+hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
+                                hipStream_t stream);
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const LevelPlan &plan, const int64_t *codes, const DenseChoice &dc, void *workspace,
-                                 hipStream_t stream);
+                                 const DenseChoice &dc, void *workspace, hipStream_t stream);
 
 }  // namespace psig

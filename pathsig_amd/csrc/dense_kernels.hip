@@ -37,6 +37,15 @@ __device__ __forceinline__ void static_for(F &&f) {
     }
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which on
+// this hardware means waiting for every outstanding global load, including prefetches that are meant to
+// stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 constexpr int ipow(int b, int e) { return e <= 0 ? 1 : b * ipow(b, e - 1); }
 // number of sub-trie values in levels 1..k below a prefix
 constexpr int trie_size(int D, int k) { return k <= 0 ? 0 : ipow(D, k) + trie_size(D, k - 1); }
@@ -159,31 +168,6 @@ struct AdjTargets {
     }
 };
 
-// ---------------------------------------------------------------------------------------------
-// wave-wide sum; the total is valid in lane 63
-// ---------------------------------------------------------------------------------------------
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add_c(float v) {
-    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false);
-    return v + __builtin_bit_cast(float, moved);
-}
-
-__device__ __forceinline__ float wave_total(float v) {
-    v = dpp_add_c<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add_c<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add_c<0x141, 0xF>(v);  // row_half_mirror
-    v = dpp_add_c<0x140, 0xF>(v);  // row_mirror: every lane now holds the sum of its row of 16
-    v = dpp_add_c<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_add_c<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
-__device__ __forceinline__ double wave_total(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
 struct Span {
     int64_t start, steps;
 };
@@ -217,7 +201,6 @@ struct Geometry {
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kFwdSub = trie_size(D, N - P);    // sub-trie levels P+1..N
     static constexpr int kASub = trie_size(D, N - 1 - P);  // levels P+1..N-1
-    static constexpr int kDumpRegs = P + kASub;            // chain + sub-trie below the top level
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
         int64_t o = 0, w = 1;
         for (int i = 1; i < k; ++i) {
@@ -266,11 +249,12 @@ __device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bo
 template <typename T, int D, int P, int TOP, int SUB>
 __device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T (&a)[P + 1], const T (&sub)[SUB]) {
     using G = Geometry<D, TOP, P>;
-    // chain values are written by the lane whose remaining prefix letters are all zero
+    // Every lane writes its chain values: lanes that share a chain node computed it with the same
+    // operations, so they store identical bits, and no branch is needed.
     int rest = 1;
 #pragma unroll
     for (int j = P; j >= 1; --j) {
-        if (pu % rest == 0) row[G::level_off(j) + pu / rest] = a[j];
+        row[G::level_off(j) + pu / rest] = a[j];
         rest *= D;
     }
     static_for<1, TOP - P + 1>([&](auto kc) {
@@ -399,7 +383,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     using G = Geometry<D, N, P>;
     __shared__ T sdx[kTile * D];
     const int pu = threadIdx.x;
-    const bool active = pu < G::kLanes;
+    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
 
@@ -422,9 +406,9 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     for (int64_t t0 = begin; t0 < end; t0 += kTile) {
         const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
         const T *xw = x + t0 * D;
-        __syncthreads();
+        lds_barrier();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
-        __syncthreads();
+        lds_barrier();
         for (int tt = 0; tt < nt; ++tt) {
             T dx[D], dxp[P];
 #pragma unroll
@@ -437,13 +421,58 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     if (active) store_state<T, D, P, N, G::kFwdSub>(out + unit * G::kSigSize, pu, a, sub);
 }
 
-// product of the chunk signatures of one row, left to right
-template <typename T, int D, int N, int P>
+// ---------------------------------------------------------------------------------------------
+// staging of one dense-layout row (COUNT elements) through registers into LDS
+// ---------------------------------------------------------------------------------------------
+// native vector types (the HIP float4 wrappers do not stay in registers as array elements)
+template <typename T, int VW>
+struct VecOf {
+    typedef T type __attribute__((ext_vector_type(VW)));
+};
+template <typename T>
+struct VecOf<T, 1> {
+    typedef T type;
+};
+
+// Rows start at multiples of COUNT elements from a 256-byte aligned base, so a row can be moved in
+// 16-byte pieces exactly when COUNT * sizeof(T) is a multiple of 16.
+template <typename T, int COUNT, int BLOCK>
+struct RowStager {
+    static constexpr int kMaxVW = 16 / (int)sizeof(T);
+    static constexpr int kVW = (COUNT % kMaxVW == 0) ? kMaxVW : ((kMaxVW == 4 && COUNT % 2 == 0) ? 2 : 1);
+    using V = typename VecOf<T, kVW>::type;
+    static constexpr int kVecs = COUNT / kVW;
+    static constexpr int kPer = (kVecs + BLOCK - 1) / BLOCK;
+    static constexpr int kPadded = kPer * BLOCK * kVW;  // elements an LDS buffer must hold
+    V regs[kPer];
+    __device__ __forceinline__ void fetch(const T *__restrict__ src) {
+        const V *v = reinterpret_cast<const V *>(src);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int idx = i * BLOCK + (int)threadIdx.x;
+            regs[i] = v[idx < kVecs ? idx : kVecs - 1];  // unconditional, so the array stays in registers
+        }
+    }
+    // dst must have room for kPadded elements: the tail of the last pass lands in the padding
+    __device__ __forceinline__ void commit(T *dst) const {
+        V *v = reinterpret_cast<V *>(dst);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) v[i * BLOCK + (int)threadIdx.x] = regs[i];
+    }
+};
+
+// product of the chunk signatures of one row, left to right.  Lanes sit on prefixes of length P (one
+// more letter than in the sweep kernels, for more lanes per row).  Chunks are fetched into registers
+// kAhead products before they are needed and handed over through a double buffer in LDS.
+template <typename T, int D, int N, int P, bool STAGED>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks) {
     using G = Geometry<D, N, P>;
+    constexpr int kStage = STAGED ? RowStager<T, (int)G::kSigSize, G::kBlock>::kPadded : 4;
+    constexpr int kAhead = 3;
+    __shared__ __align__(16) T sB[2][kStage];
     const int pu = threadIdx.x;
-    const bool active = pu < G::kLanes;
+    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
     const SubWords<D, P> sw(u);
@@ -452,39 +481,44 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     T a[P + 1];
     T sub[G::kFwdSub];
     load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
-    for (int c = 1; c < chunks; ++c) apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
+    if constexpr (STAGED) {
+        // Register set q holds chunk c with (c - 1) % kAhead == q.  Fetches past the last chunk re-read the
+        // last chunk instead of branching, so the waits on them stay exact counts.
+        const int last = chunks - 1;
+        RowStager<T, (int)G::kSigSize, G::kBlock> stager[kAhead];
+        static_for<0, kAhead>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            stager[q].fetch(rows + (int64_t)(1 + q < last ? 1 + q : last) * G::kSigSize);
+        });
+        stager[0].commit(sB[1]);
+        stager[0].fetch(rows + (int64_t)(1 + kAhead < last ? 1 + kAhead : last) * G::kSigSize);
+        lds_barrier();
+        for (int base = 1; base < chunks; base += kAhead) {
+            static_for<0, kAhead>([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                constexpr int qn = (q + 1) % kAhead;  // register set of the next chunk
+                const int c = base + q;
+                if (c < chunks) {
+                    apply_right<T, D, P, N, G::kFwdSub>(a, sub, sB[c & 1], sw);
+                    stager[qn].commit(sB[(c + 1) & 1]);
+                    const int nxt = c + 1 + kAhead;
+                    stager[qn].fetch(rows + (int64_t)(nxt < last ? nxt : last) * G::kSigSize);
+                    lds_barrier();
+                }
+            });
+        }
+    } else {
+        for (int c = 1; c < chunks; ++c)
+            apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
+    }
     if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
 }
 
 // ---------------------------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------------------------
-// Register dump of a lane's chain + sub-trie below the top level: element (reg, lane) of unit at
-// ((unit * kDumpRegs) + reg) * kBlock + lane.
-template <typename T, int D, int N, int P, int SUBN>
-__device__ __forceinline__ void dump_state(T *__restrict__ dst, int64_t unit, int lane, const T (&c)[P + 1],
-                                           const T (&sub)[SUBN]) {
-    using G = Geometry<D, N, P>;
-    T *base = dst + unit * G::kDumpRegs * G::kBlock + lane;
-#pragma unroll
-    for (int j = 1; j <= P; ++j) base[(j - 1) * G::kBlock] = c[j];
-#pragma unroll
-    for (int i = 0; i < G::kASub; ++i) base[(P + i) * G::kBlock] = sub[i];
-}
-
-template <typename T, int D, int N, int P, int SUBN>
-__device__ __forceinline__ void undump_state(const T *__restrict__ src, int64_t unit, int lane, T (&c)[P + 1],
-                                             T (&sub)[SUBN]) {
-    using G = Geometry<D, N, P>;
-    const T *base = src + unit * G::kDumpRegs * G::kBlock + lane;
-#pragma unroll
-    for (int j = 1; j <= P; ++j) c[j] = base[(j - 1) * G::kBlock];
-#pragma unroll
-    for (int i = 0; i < G::kASub; ++i) sub[i] = base[(P + i) * G::kBlock];
-}
-
-// initial adjoint state of a row: chain entries are lane-private partial sums, so only the lane whose
-// remaining prefix letters are zero starts from the upstream gradient
+// Adjoint state of a lane at the right end of a row: the upstream gradient.  Chain entries are
+// lane-private partial sums, so only the lane whose remaining prefix letters are zero starts from it.
 template <typename T, int D, int N, int P>
 __device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu, bool active, T (&hc)[P + 1],
                                              T (&hsub)[Geometry<D, N, P>::kFwdSub]) {
@@ -499,46 +533,95 @@ __device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu,
     hc[0] = T(0);
 }
 
-// Per row: state at the right edge of every chunk.  blockIdx.y == 0: A_c = S_0 (x) .. (x) S_c (levels < N),
-// blockIdx.y == 1: H_c = adjoint of the signature at the right edge of chunk c.
+// Per row, from the chunk signatures S_c (levels 1..N-1, dense-layout rows): the signature up to the
+// right edge of every chunk, and the signature from there to the end of the row.
+//   blockIdx.y == 0:  edgeA_c = S_0 (x) .. (x) S_c            (state in registers, multiplied on the right)
+//   blockIdx.y == 1:  edgeZ_c = S_{c+1} (x) .. (x) S_{C-1}      (state in LDS, multiplied on the left:
+//                     the lanes load S_c as their state and multiply it by the running product)
+// Chunk signatures pass through a double buffer in LDS.  The first kBlock threads do the algebra and
+// only ever wait on their own prefetches; the results of a round are left in LDS and copied to global
+// memory during the next round by kCopyThreads extra threads, whose stores nobody waits for.
+constexpr int kCopyThreads = 128;
+
+template <typename T, int COUNT>
+__device__ __forceinline__ void copy_row_out(const T *src_lds, T *__restrict__ dst, int tid) {
+    for (int idx = tid; idx < COUNT; idx += kCopyThreads) dst[idx] = src_lds[idx];
+}
+
 template <typename T, int D, int N, int P>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
-    dense_scan_kernel(const T *__restrict__ chunk_low, const T *__restrict__ grad_sig, T *__restrict__ dumpA,
-                      T *__restrict__ dumpH, int chunks) {
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
+    dense_scan_kernel(const T *__restrict__ chunk_low, T *__restrict__ edgeA, T *__restrict__ edgeZ, int chunks) {
     using G = Geometry<D, N, P>;
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
-    const int pu = threadIdx.x;
-    const bool active = pu < G::kLanes;
+    constexpr int kLow = (int)G::kLowSize;
+    __shared__ __align__(16) T sB[2][RowStager<T, kLow, G::kBlock>::kPadded];
+    __shared__ __align__(16) T sOut[2][kLow];
+    const bool copier = threadIdx.x >= G::kBlock;
+    const int ctid = (int)threadIdx.x - G::kBlock;
+    const int pu = copier ? 0 : (int)threadIdx.x;
+    const bool active = !copier && ((G::kLanes == G::kBlock) || pu < G::kLanes);
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
     const SubWords<D, P> sw(u);
     const int64_t row = blockIdx.x;
-    const T *rows = chunk_low + row * chunks * G::kLowSize;
+    const T *rows = chunk_low + row * chunks * kLow;
+    RowStager<T, kLow, G::kBlock> stager;
+    T a[P + 1];
+    T asub[kAS];
+    const int last = chunks - 1;
     if (blockIdx.y == 0) {
-        T a[P + 1];
-        T asub[kAS];
-        load_state<T, D, P, N - 1, kAS>(rows, pu, active, a, asub);
-        dump_state<T, D, N, P, kAS>(dumpA, row * chunks, pu, a, asub);
+        T *edge = edgeA + row * chunks * kLow;
+        if (!copier) {
+            load_state<T, D, P, N - 1, kAS>(rows, pu, active, a, asub);
+            stager.fetch(rows + (int64_t)(1 < last ? 1 : last) * kLow);
+            stager.commit(sB[1]);
+            stager.fetch(rows + (int64_t)(2 < last ? 2 : last) * kLow);
+            if (active) store_state<T, D, P, N - 1, kAS>(sOut[0], pu, a, asub);
+        }
+        lds_barrier();
         for (int c = 1; c < chunks; ++c) {
-            apply_right<T, D, P, N - 1, kAS>(a, asub, rows + (int64_t)c * G::kLowSize, sw);
-            dump_state<T, D, N, P, kAS>(dumpA, row * chunks + c, pu, a, asub);
+            if (!copier) {
+                apply_right<T, D, P, N - 1, kAS>(a, asub, sB[c & 1], sw);
+                stager.commit(sB[(c + 1) & 1]);
+                stager.fetch(rows + (int64_t)(c + 2 < last ? c + 2 : last) * kLow);
+                if (active) store_state<T, D, P, N - 1, kAS>(sOut[c & 1], pu, a, asub);
+            } else {
+                copy_row_out<T, kLow>(sOut[(c - 1) & 1], edge + (int64_t)(c - 1) * kLow, ctid);
+            }
+            lds_barrier();
         }
+        if (copier) copy_row_out<T, kLow>(sOut[last & 1], edge + (int64_t)last * kLow, ctid);
     } else {
-        T hc[P + 1];
-        T hsub[G::kFwdSub];
-        load_adjoint<T, D, N, P>(grad_sig + row * G::kSigSize, pu, active, hc, hsub);
-        dump_state<T, D, N, P, G::kFwdSub>(dumpH, row * chunks + chunks - 1, pu, hc, hsub);
-        for (int c = chunks - 1; c >= 1; --c) {
-            contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, rows + (int64_t)c * G::kLowSize, sw);
-            dump_state<T, D, N, P, G::kFwdSub>(dumpH, row * chunks + c - 1, pu, hc, hsub);
+        T *edge = edgeZ + row * chunks * kLow;
+        // the product to the right of the last chunk is the identity (all coefficients zero)
+        if (!copier) {
+            for (int idx = threadIdx.x; idx < kLow; idx += G::kBlock) sOut[last & 1][idx] = T(0);
+            stager.fetch(rows + (int64_t)last * kLow);
+            stager.commit(sB[last & 1]);
+            stager.fetch(rows + (int64_t)(last - 1 > 0 ? last - 1 : 0) * kLow);
         }
+        lds_barrier();
+        for (int c = last; c >= 1; --c) {
+            if (!copier) {
+                // Z_{c-1} = S_c (x) Z_c
+                load_state<T, D, P, N - 1, kAS>(sB[c & 1], pu, active, a, asub);
+                apply_right<T, D, P, N - 1, kAS>(a, asub, sOut[c & 1], sw);
+                if (active) store_state<T, D, P, N - 1, kAS>(sOut[(c - 1) & 1], pu, a, asub);
+                stager.commit(sB[(c - 1) & 1]);
+                stager.fetch(rows + (int64_t)(c - 2 > 0 ? c - 2 : 0) * kLow);
+            } else {
+                copy_row_out<T, kLow>(sOut[c & 1], edge + (int64_t)c * kLow, ctid);
+            }
+            lds_barrier();
+        }
+        if (copier) copy_row_out<T, kLow>(sOut[0], edge, ctid);
     }
 }
 
 template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
-                          const T *__restrict__ dumpA, const T *__restrict__ dumpH, T *__restrict__ grad_inc,
+                          const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
                           SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
     __shared__ T sdx[kTile * D];
@@ -546,7 +629,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     const int pu = threadIdx.x;
     const int lane = pu & (kWave - 1);
     const int wave = pu / kWave;
-    const bool active = pu < G::kLanes;
+    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
 
@@ -568,8 +651,11 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     T hsub[G::kFwdSub];
     load_adjoint<T, D, N, P>(grow, pu, active, hc, hsub);
     if constexpr (CHUNKED) {
-        undump_state<T, D, N, P, kAS>(dumpA, unit, pu, a, asub);
-        undump_state<T, D, N, P, G::kFwdSub>(dumpH, unit, pu, hc, hsub);
+        load_state<T, D, P, N - 1, kAS>(edgeA + unit * G::kLowSize, pu, active, a, asub);
+        // adjoint at the right edge of the chunk: the upstream gradient contracted with the signature of
+        // everything to the right of the chunk
+        const SubWords<D, P> sw(u);
+        contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
     } else {
         load_state<T, D, P, N - 1, kAS>(sig + row * G::kSigSize, pu, active, a, asub);
     }
@@ -581,9 +667,9 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
         const int64_t t0 = begin + ti * kTile;
         const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
         const T *xw = x + t0 * D;
-        __syncthreads();
+        lds_barrier();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
-        __syncthreads();
+        lds_barrier();
         for (int tt = nt - 1; tt >= 0; --tt) {
             T dx[D], dxp[P];
 #pragma unroll
@@ -608,7 +694,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                 if (lane == kWave - 1) sg[wave][tt * D + k] = v;
             }
         }
-        __syncthreads();
+        lds_barrier();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
             T v = sg[0][idx];
 #pragma unroll
@@ -625,22 +711,26 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 // ---------------------------------------------------------------------------------------------
 // host side: table of compiled shapes and launch sequences
 // ---------------------------------------------------------------------------------------------
-// X(index, D, N, P): signature over D letters to depth N with lanes on prefixes of length P.  The
-// backward also runs the forward kernel of depth N-1 (same P) to get chunk signatures below the top level.
-#define PSIG_VARIANTS(X) X(0, 4, 6, 3) X(1, 8, 4, 2) X(2, 6, 5, 3) X(3, 4, 4, 2) X(4, 3, 5, 3) X(5, 2, 8, 5)
+// X(index, D, N, P, PC, PS): signature over D letters to depth N; the sweep kernels put lanes on prefixes
+// of length P, the per-row combine kernel on prefixes of length PC and the per-row scan kernel (which
+// works on levels below N) on prefixes of length PS.  The backward also runs the forward kernel of
+// depth N-1 (same P) to get chunk signatures below the top level.
+#define PSIG_VARIANTS(X) \
+    X(0, 4, 6, 3, 5, 4) X(1, 8, 4, 2, 3, 2) X(2, 6, 5, 3, 3, 3) X(3, 4, 4, 2, 3, 2) X(4, 3, 5, 3, 4, 3) \
+    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3)
 
 struct VariantInfo {
-    int d, depth, block, dump_regs;
+    int d, depth, block;
     int64_t sig_size, low_size;
 };
 
 template <int D, int N, int P>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
-    return VariantInfo{D, N, G::kBlock, G::kDumpRegs, G::kSigSize, G::kLowSize};
+    return VariantInfo{D, N, G::kBlock, G::kSigSize, G::kLowSize};
 }
 
-#define PSIG_INFO(I, D, N, P) variant_info<D, N, P>(),
+#define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P>(),
 constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
 #undef PSIG_INFO
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -660,9 +750,11 @@ int pick_chunks(int64_t rows, int block, int64_t L) {
     return (int)c;
 }
 
-template <typename T, int D, int N, int P>
+template <typename T, int D, int N, int P, int PC>
 hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
+    using GC = Geometry<D, N, PC>;
+    constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
     const int64_t rows = shape.B * shape.W;
     if (chunks <= 1) {
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream, path,
@@ -674,15 +766,16 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                        path, chunk_sig, shape, chunks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((dense_combine_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
+    hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, kStaged>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
                        (const T *)chunk_sig, sig, chunks);
     return hipGetLastError();
 }
 
-template <typename T, int D, int N, int P>
+template <typename T, int D, int N, int P, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape, int chunks,
                         void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
+    using GC = Geometry<D, N, PS>;
     const int64_t rows = shape.B * shape.W;
     const bool accumulate = shape.windows != nullptr;
     hipError_t e;
@@ -710,15 +803,15 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         T *chunk_low = (T *)ws;
         ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpA = (T *)ws;
-        ws += pad256((size_t)units * G::kDumpRegs * G::kBlock * sizeof(T));
+        ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpH = (T *)ws;
         // chunk signatures below the top level: the depth N-1 forward kernel on the same units
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P>), dim3((unsigned)units),
                            dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL((dense_scan_kernel<T, D, N, P>), dim3((unsigned)rows, 2), dim3(G::kBlock), 0, stream,
-                           (const T *)chunk_low, grad_sig, dumpA, dumpH, chunks);
+        hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS>), dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), 0, stream,
+                           (const T *)chunk_low, dumpA, dumpH, chunks);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         if (accumulate)
@@ -735,42 +828,53 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
 
 }  // namespace
 
-DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *, int64_t B, int64_t L,
-                         int64_t W, bool) {
-    DenseChoice dc{false, -1, 1, 0, 0};
-    if (!all_dense || B <= 0 || W <= 0) return dc;
+DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,
+                         int64_t L, int64_t W, bool) {
+    DenseChoice dc{};
+    dc.variant = -1;
+    dc.fwd_chunks = dc.bwd_chunks = 1;
+    if (B <= 0 || W <= 0) return dc;
     for (int i = 0; i < kNumVariants; ++i) {
         const VariantInfo &v = kVariants[i];
         if (v.d != d || v.depth != depth) continue;
         const int64_t rows = B * W;
+        if (!all_dense) {
+            // A word projection is worth computing densely when its top level keeps a fair share of the
+            // words (the top level dominates the cost) and the dense rows fit comfortably in memory.
+            if (!level_sizes) return dc;
+            const int64_t top_dense = v.sig_size - v.low_size;
+            if (level_sizes[depth] * 8 < top_dense) return dc;
+            if ((double)rows * (double)v.sig_size * (double)elem > 4e9) return dc;
+            dc.embed = true;
+            dc.dense_bytes = pad256((size_t)rows * v.sig_size * elem);
+        }
         int chunks = pick_chunks(rows, v.block, L);
         if (const char *env = getenv("PATHSIG_CHUNKS")) {
             const int forced = atoi(env);
             if (forced >= 1 && forced <= 1024) chunks = forced;
         }
-        if (rows * chunks >= (int64_t(1) << 31)) return dc;
+        if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
         dc.variant = i;
-        dc.chunks = chunks;
-        if (chunks > 1) {
-            const size_t units = (size_t)rows * chunks;
-            dc.forward_workspace = pad256(units * v.sig_size * elem);
-            dc.backward_workspace = pad256(units * v.low_size * elem) +
-                                    2 * pad256(units * (size_t)v.dump_regs * v.block * elem);
-        }
+        dc.fwd_chunks = chunks;
+        dc.bwd_chunks = (dc.embed && chunks < 2) ? 2 : chunks;
+        dc.forward_workspace = dc.dense_bytes;
+        dc.backward_workspace = dc.dense_bytes;
+        if (dc.fwd_chunks > 1) dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem);
+        if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
         return dc;
     }
     return dc;
 }
 
-#define PSIG_CASE_FWD(I, D, N, P) \
-    case I: return run_forward<T, D, N, P>(path, sig, shape, dc.chunks, workspace, stream);
-#define PSIG_CASE_BWD(I, D, N, P) \
-    case I: return run_backward<T, D, N, P>(path, sig, grad_sig, grad_inc, shape, dc.chunks, workspace, stream);
+#define PSIG_CASE_FWD(I, D, N, P, PC, PS) \
+    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, workspace, stream);
+#define PSIG_CASE_BWD(I, D, N, P, PC, PS) \
+    case I: return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, shape, dc.bwd_chunks, workspace, stream);
 
 template <typename T>
-hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const LevelPlan &, const int64_t *,
-                                const DenseChoice &dc, void *workspace, hipStream_t stream) {
+hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
+                                hipStream_t stream) {
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_FWD)
         default: return hipErrorNotSupported;
@@ -779,20 +883,18 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
 
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const LevelPlan &, const int64_t *, const DenseChoice &dc, void *workspace,
-                                 hipStream_t stream) {
+                                 const DenseChoice &dc, void *workspace, hipStream_t stream) {
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_BWD)
         default: return hipErrorNotSupported;
     }
 }
 
-#define PSIG_INSTANTIATE(T)                                                                                  \
-    template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const LevelPlan &,         \
-                                                const int64_t *, const DenseChoice &, void *, hipStream_t);  \
-    template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, const SigShape &,     \
-                                                 const LevelPlan &, const int64_t *, const DenseChoice &,    \
-                                                 void *, hipStream_t);
+#define PSIG_INSTANTIATE(T)                                                                                    \
+    template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const DenseChoice &, void *,  \
+                                                hipStream_t);                                                  \
+    template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, const SigShape &,       \
+                                                 const DenseChoice &, void *, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE

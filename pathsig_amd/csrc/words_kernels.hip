@@ -20,6 +20,7 @@ namespace psig {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr int kLetterLoopMax = 32;  // path dimensions up to this use one wave-wide sum per letter in the backward
 
 template <typename T>
 __device__ __forceinline__ T fma_t(T a, T b, T c);
@@ -226,7 +227,7 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
             sacc[idx] = T(0);
         }
         __syncthreads();
-        if (active || uniform_mask) {
+        if (active || uniform_mask || d <= kLetterLoopMax) {
             for (int tt = nt - 1; tt >= 0; --tt) {
                 const T *dxr = sdx + (int64_t)tt * d;
                 T *acc = sacc + (int64_t)tt * d;
@@ -257,13 +258,25 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
                         }
                     }
                 }
+                if (d <= kLetterLoopMax) {
+                    // few letters: one wave-wide sum per letter, then a single lane adds it to the tile
+                    // accumulator (many lanes adding to the same LDS word would serialise badly)
+                    for (int letter = 0; letter < (int)d; ++letter) {
+                        T v = T(0);
 #pragma unroll
-                for (int k = 0; k < DEG; ++k) {
-                    if (uniform_mask & (1u << k)) {
-                        const T v = wave_sum<T>(gl[k]);
-                        if (lane == 0 && v != T(0)) atomicAdd(&acc[l[k]], v);
-                    } else if (gl[k] != T(0)) {
-                        atomicAdd(&acc[l[k]], gl[k]);
+                        for (int k = 0; k < DEG; ++k) v += (l[k] == letter) ? gl[k] : T(0);
+                        v = wave_total(v);
+                        if (lane == kWave - 1 && v != T(0)) atomicAdd(&acc[letter], v);
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < DEG; ++k) {
+                        if (uniform_mask & (1u << k)) {
+                            const T v = wave_sum<T>(gl[k]);
+                            if (lane == 0 && v != T(0)) atomicAdd(&acc[l[k]], v);
+                        } else if (gl[k] != T(0)) {
+                            atomicAdd(&acc[l[k]], gl[k]);
+                        }
                     }
                 }
             }
@@ -324,6 +337,65 @@ __global__ void increments_to_path_kernel(const T *__restrict__ ginc, T *__restr
     }
 }
 
+// Column j of the projected layout <-> its column in the dense layout (same rule as the forward
+// kernels: dense levels map to themselves, listed levels go through their codes).
+struct ColumnMap {
+    int depth;
+    int64_t out_off[kMaxDepth + 2];    // first projected column of level k; [depth+1] = projected size
+    int64_t code_off[kMaxDepth + 1];   // offset into the code array, < 0 for dense levels
+    int64_t dense_off[kMaxDepth + 1];  // first dense column of level k
+    int64_t dense_size;
+};
+
+__device__ __forceinline__ int64_t dense_column(const ColumnMap &m, const int64_t *__restrict__ codes, int64_t col) {
+    int k = 1;
+    while (k < m.depth && col >= m.out_off[k + 1]) ++k;
+    const int64_t j = col - m.out_off[k];
+    const int64_t code = m.code_off[k] >= 0 ? codes[m.code_off[k] + j] : j;
+    return m.dense_off[k] + code;
+}
+
+template <typename T>
+__global__ void gather_columns_kernel(const T *__restrict__ dense, T *__restrict__ out, ColumnMap m,
+                                      const int64_t *__restrict__ codes, int64_t rows) {
+    const int64_t width = m.out_off[m.depth + 1];
+    const int64_t total = rows * width;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t row = i / width;
+        out[i] = dense[row * m.dense_size + dense_column(m, codes, i - row * width)];
+    }
+}
+
+// dense must be zero on entry; repeated columns add up
+template <typename T>
+__global__ void scatter_columns_kernel(const T *__restrict__ grad, T *__restrict__ dense, ColumnMap m,
+                                       const int64_t *__restrict__ codes, int64_t rows) {
+    const int64_t width = m.out_off[m.depth + 1];
+    const int64_t total = rows * width;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t row = i / width;
+        atomicAdd(&dense[row * m.dense_size + dense_column(m, codes, i - row * width)], grad[i]);
+    }
+}
+
+ColumnMap make_column_map(const LevelPlan &plan, int64_t d) {
+    ColumnMap m{};
+    m.depth = plan.depth;
+    int64_t off = 0, width = 1;
+    for (int k = 1; k <= plan.depth; ++k) {
+        width *= d;
+        m.out_off[k] = plan.out_off[k];
+        m.code_off[k] = plan.code_off[k];
+        m.dense_off[k] = off;
+        off += width;
+    }
+    m.out_off[plan.depth + 1] = plan.sig_size;
+    m.dense_size = off;
+    return m;
+}
+
 int pick_tile(int64_t d, size_t elem, int64_t max_steps, int arrays) {
     const int64_t budget = 16384 / arrays;
     int64_t tile = budget / (int64_t)(d * elem);
@@ -382,7 +454,35 @@ hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B,
     return hipGetLastError();
 }
 
+template <typename T>
+hipError_t launch_gather_columns(const T *dense, T *out, const LevelPlan &plan, int64_t d, const int64_t *codes,
+                                 int64_t rows, hipStream_t stream) {
+    const int64_t n = rows * plan.sig_size;
+    if (n <= 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(gather_columns_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, dense, out,
+                       make_column_map(plan, d), codes, rows);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan, int64_t d, const int64_t *codes,
+                                  int64_t rows, hipStream_t stream) {
+    const int64_t n = rows * plan.sig_size;
+    if (n <= 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(scatter_columns_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad, dense,
+                       make_column_map(plan, d), codes, rows);
+    return hipGetLastError();
+}
+
 #define PSIG_INSTANTIATE(T)                                                                                         \
+    template hipError_t launch_gather_columns<T>(const T *, T *, const LevelPlan &, int64_t, const int64_t *,       \
+                                                 int64_t, hipStream_t);                                             \
+    template hipError_t launch_scatter_columns<T>(const T *, T *, const LevelPlan &, int64_t, const int64_t *,      \
+                                                  int64_t, hipStream_t);                                            \
     template hipError_t launch_words_forward<T>(const T *, T *, const SigShape &, const LevelPlan &, const int64_t *, \
                                                 hipStream_t);                                                       \
     template hipError_t launch_words_backward<T>(const T *, const T *, const T *, T *, const SigShape &,            \

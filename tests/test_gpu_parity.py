@@ -311,3 +311,48 @@ def test_tiled_shapes_time_chunked_windows(ps, monkeypatch, d, depth):
     got, grad = _run_sig(ps, path, depth, torch.float64, windows=wins, G=G)
     assert rel_err(got, want) < 1e-12
     assert rel_err(grad, TO.signature_vjp(path, G, depth, windows=wins)) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------
+# word projections that are computed through the dense kernels and gathered (top level kept >= 1/8)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,kind", [(4, 4, "lyndon"), (3, 5, "lyndon"), (4, 4, "words"), (3, 5, "dups")])
+def test_projection_through_dense_kernels(ps, dtype, d, depth, kind):
+    B, L = 3, 70
+    if kind == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    elif kind == "words":
+        words = random_word_set(d, 1, depth - 1, 30, seed=9) + [w for w in random_word_set(d, depth, depth, 80, seed=10)]
+        proj = ps.projections.words(words, depth=depth, path_dim=d)
+    else:  # repeated words: their gradients must add up
+        top = random_word_set(d, depth, depth, 40, seed=11)
+        proj = ps.projections.words([(0,), (2,), (0,), (1, 1), (1, 1)] + top + top[:7], depth=depth, path_dim=d)
+    sizes, codes = _plan(proj)
+    assert sizes[depth] * 8 >= d ** depth
+    path = brownian_path(B, L, d, seed=71)
+    wins = [(0, 70), (5, 40), (33, 35)]
+    for windows in (None, wins):
+        want = TO.compute_signature(path, depth, sizes, codes, windows)
+        G = randn(tuple(want.shape), seed=72)
+        got, grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[dtype]
+        want_grad = TO.signature_vjp(path, G, depth, sizes, codes, windows)
+        assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_logsignature_lyndon_through_dense_kernels(ps, dtype):
+    d, depth, B, L = 4, 4, 3, 60
+    proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    path = brownian_path(B, L, d, seed=73)
+    cols = torch.tensor(TO.projection_columns(d, depth, proj.level_sizes, proj._codes))
+    want = TO.logsignature(path, depth).index_select(-1, cols)
+    G = randn(tuple(want.shape), seed=74)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    out = ps.LogSignature(depth=depth, projection=proj)(x)
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    assert rel_err(out.detach(), want) < TOL[dtype]
+    xr = path.clone().requires_grad_(True)
+    (want_grad,) = torch.autograd.grad(TO.logsignature(xr, depth).index_select(-1, cols), xr, G)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
