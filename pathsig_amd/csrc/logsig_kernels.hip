@@ -98,9 +98,33 @@ __global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__re
     }
 }
 
+// Accumulators of the adjoint.  Short words collect contributions from every longer word, so the
+// columns below `lds_cols` (whole levels) live in LDS, where the adds are cheap; the rest are global.
+template <typename T>
+struct AdjointSink {
+    T *gs;         // global: gradient w.r.t. the signature, one row
+    T *gP;         // global: adjoint of the power cache, rows of `depth`, levels below the top
+    T *lds_gs;     // LDS copies of the first lds_cols columns
+    T *lds_gP;
+    int64_t lds_cols;
+    int depth;
+    __device__ __forceinline__ void add_gs(uint64_t col, T v) {
+        if ((int64_t)col < lds_cols) atomicAdd(&lds_gs[col], v);
+        else atomicAdd(&gs[col], v);
+    }
+    __device__ __forceinline__ void add_gP(uint64_t col, int m_index, T v) {
+        if ((int64_t)col < lds_cols) atomicAdd(&lds_gP[col * depth + m_index], v);
+        else atomicAdd(&gP[col * depth + m_index], v);
+    }
+    __device__ __forceinline__ T read_gP(uint64_t col, int m_index) const {
+        return ((int64_t)col < lds_cols) ? lds_gP[col * depth + m_index] : gP[col * depth + m_index];
+    }
+};
+
 template <typename T, int DEG>
 __device__ void logsig_backward_level(const T *__restrict__ s, const T *__restrict__ P, const T *__restrict__ gl,
-                                      T *gs, T *gP, const HybridPlan &hp, const int64_t *__restrict__ top_words) {
+                                      AdjointSink<T> &sink, const HybridPlan &hp,
+                                      const int64_t *__restrict__ top_words) {
     const int depth = hp.depth;
     const uint64_t d = (uint64_t)hp.d;
     const bool top = (DEG == depth);
@@ -128,17 +152,17 @@ __device__ void logsig_backward_level(const T *__restrict__ s, const T *__restri
 #pragma unroll
         for (int m = 1; m <= DEG; ++m) {
             // a top-level word is nobody's prefix: nothing has been accumulated for it
-            const T acc = top ? T(0) : gP[own * (uint64_t)depth + (uint64_t)(m - 1)];
+            const T acc = top ? T(0) : sink.read_gP(own, m - 1);
             gPv[m - 1] = alt_coeff<T>(m) * g + acc;
         }
-        atomicAdd(&gs[own], gPv[0]);
+        sink.add_gs(own, gPv[0]);
 #pragma unroll
         for (int m = 2; m <= DEG; ++m) {
 #pragma unroll
             for (int k = m - 1; k < DEG; ++k) {
                 const uint64_t pi = pidx[k], si = sidx[DEG - k];
-                atomicAdd(&gP[pi * (uint64_t)depth + (uint64_t)(m - 2)], gPv[m - 1] * s[si]);
-                atomicAdd(&gs[si], gPv[m - 1] * P[pi * (uint64_t)depth + (uint64_t)(m - 2)]);
+                sink.add_gP(pi, m - 2, gPv[m - 1] * s[si]);
+                sink.add_gs(si, gPv[m - 1] * P[pi * (uint64_t)depth + (uint64_t)(m - 2)]);
             }
         }
     }
@@ -148,21 +172,29 @@ template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__restrict__ sig, const T *__restrict__ P,
                                                                     const T *__restrict__ grad_logsig, T *grad_sig,
                                                                     T *gradP, HybridPlan hp,
-                                                                    const int64_t *__restrict__ top_words) {
+                                                                    const int64_t *__restrict__ top_words,
+                                                                    int64_t lds_cols) {
+    extern __shared__ __align__(16) unsigned char logsig_smem[];
     const int64_t row = blockIdx.x;
     const T *s = sig + row * hp.total;
     const T *Pr = P + row * hp.total * hp.depth;
     const T *gl = grad_logsig + row * hp.total;
-    T *gs = grad_sig + row * hp.total;
-    T *gP = gradP + row * hp.lower * hp.depth;
-    for (int64_t i = threadIdx.x; i < hp.total; i += kLogBlock) gs[i] = T(0);
-    for (int64_t i = threadIdx.x; i < hp.lower * hp.depth; i += kLogBlock) gP[i] = T(0);
+    AdjointSink<T> sink;
+    sink.gs = grad_sig + row * hp.total;
+    sink.gP = gradP + row * hp.lower * hp.depth;
+    sink.lds_gs = reinterpret_cast<T *>(logsig_smem);
+    sink.lds_gP = sink.lds_gs + lds_cols;
+    sink.lds_cols = lds_cols;
+    sink.depth = hp.depth;
+    for (int64_t i = threadIdx.x; i < hp.total; i += kLogBlock) sink.gs[i] = T(0);
+    for (int64_t i = threadIdx.x; i < hp.lower * hp.depth; i += kLogBlock) sink.gP[i] = T(0);
+    for (int64_t i = threadIdx.x; i < lds_cols * (hp.depth + 1); i += kLogBlock) sink.lds_gs[i] = T(0);
     __threadfence_block();
     __syncthreads();
     for (int deg = hp.depth; deg >= 1; --deg) {
         switch (deg) {
 #define PSIG_CASE(N) \
-    case N: logsig_backward_level<T, N>(s, Pr, gl, gs, gP, hp, top_words); break;
+    case N: logsig_backward_level<T, N>(s, Pr, gl, sink, hp, top_words); break;
             PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
             PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
 #undef PSIG_CASE
@@ -171,6 +203,18 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
         __threadfence_block();
         __syncthreads();
     }
+    for (int64_t i = threadIdx.x; i < lds_cols; i += kLogBlock) sink.gs[i] = sink.lds_gs[i];
+}
+
+// largest number of whole low levels whose accumulators (1 + depth values per column) fit `budget` bytes
+int64_t lds_columns(int64_t d, int depth, size_t elem, size_t budget) {
+    int64_t cols = 0, width = 1;
+    for (int k = 1; k < depth; ++k) {
+        width *= d;
+        if ((size_t)(cols + width) * (size_t)(depth + 1) * elem > budget) break;
+        cols += width;
+    }
+    return cols;
 }
 
 HybridPlan make_hybrid(int64_t d, int depth, int64_t top_size, const int64_t *top_words) {
@@ -210,8 +254,10 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
                                   hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
     const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
-    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, P, grad_logsig,
-                       grad_sig, gradP, hp, top_words);
+    const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
+    const size_t lds_bytes = (size_t)lds_cols * (size_t)(depth + 1) * sizeof(T);
+    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), lds_bytes, stream, sig, P,
+                       grad_logsig, grad_sig, gradP, hp, top_words, lds_cols);
     return hipGetLastError();
 }
 
