@@ -1,0 +1,80 @@
+"""The C ABI without a GPU: the library loads, exports every function that include/pathsig_hip.h declares,
+and rejects bad arguments with its error codes before anything is launched."""
+from __future__ import annotations
+
+import ctypes
+import pathlib
+import re
+
+import pytest
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "pathsig_hip.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from pathsig_amd import _load
+    return _load.lib()
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(pathsig_[a-z_]+)\s*\(", text)))
+
+
+def test_header_functions_are_exported(lib):
+    names = declared_functions()
+    assert {"pathsig_sig_forward", "pathsig_sig_backward", "pathsig_logsig_forward", "pathsig_logsig_backward",
+            "pathsig_sig_forward_workspace", "pathsig_sig_backward_workspace", "pathsig_logsig_backward_workspace",
+            "pathsig_last_error", "pathsig_abi_version"} <= set(names)
+    for name in names:
+        assert hasattr(lib, name), name
+    assert lib.pathsig_abi_version() == 1
+
+
+def _fwd(lib, dtype=0, B=2, L=5, d=3, depth=3, path=1, sig=1, sizes=None):
+    arr = None if sizes is None else (ctypes.c_int64 * len(sizes))(*sizes)
+    return lib.pathsig_sig_forward(ctypes.c_void_p(path), ctypes.c_void_p(sig), dtype, B, L, d, depth, arr, None, 0,
+                                   None, 0, None, 0, None)
+
+
+def test_argument_errors_have_codes_and_messages(lib):
+    ERR_ARG, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3
+    assert _fwd(lib, depth=0) == ERR_ARG and b"depth" in lib.pathsig_last_error()
+    assert _fwd(lib, depth=13) == ERR_ARG
+    assert _fwd(lib, dtype=7) == ERR_ARG and b"dtype" in lib.pathsig_last_error()
+    assert _fwd(lib, L=1) == ERR_ARG and b"2 time steps" in lib.pathsig_last_error()
+    assert _fwd(lib, d=0) == ERR_ARG
+    assert _fwd(lib, path=0) == ERR_ARG and b"NULL" in lib.pathsig_last_error()
+    assert _fwd(lib, d=5000) == ERR_UNSUPPORTED
+    # a projection whose level sizes need codes, but no code array
+    assert _fwd(lib, sizes=[0, 3, 2, 0]) == ERR_ARG and b"encoded_words" in lib.pathsig_last_error()
+    assert _fwd(lib, sizes=[0, 3, -1, 0]) == ERR_ARG
+    # backward without its workspace
+    rc = lib.pathsig_sig_backward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0,
+                                  2, 5, 3, 3, None, None, 0, None, 0, None, 0, None)
+    assert rc == ERR_WORKSPACE and b"workspace" in lib.pathsig_last_error()
+    # log-signature entry points
+    assert lib.pathsig_logsig_forward(None, None, None, 0, 4, 3, 3, 27, None, None) == ERR_ARG
+    assert lib.pathsig_logsig_forward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0, 4, 3, 3, 5, None,
+                                      None) == ERR_ARG  # listed top level without its codes
+    assert lib.pathsig_logsig_forward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0, 4, 3, 0, 0, None,
+                                      None) == ERR_ARG
+    # empty batches are a no-op
+    assert _fwd(lib, B=0, path=0, sig=0) == 0
+    assert lib.pathsig_logsig_forward(None, None, None, 0, 0, 3, 3, 27, None, None) == 0
+
+
+def test_workspace_sizes(lib):
+    # general kernels: the forward needs none, the backward one increment accumulator
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 5, 3, None, 0) == 0
+    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 5, 3, None, 0)
+    assert need >= 4 * 99 * 5 * 4
+    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 5, 3, None, 0) >= 4 * 99 * 5 * 8
+    # a long path on a tiled shape is cut into chunks, which need scratch in the forward too
+    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, None, 0) > 0
+    assert lib.pathsig_sig_forward_workspace(0, 4096, 64, 4, 6, None, 0) == 0
+    assert lib.pathsig_logsig_backward_workspace(0, 10, 3, 4, 81) >= 10 * (3 + 9 + 27) * 4 * 4
+    # bad arguments give 0
+    assert lib.pathsig_sig_forward_workspace(0, 4, 1, 5, 3, None, 0) == 0
