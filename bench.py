@@ -202,6 +202,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also copy one 256 MiB buffer once (untimed), as the known-size kernel that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
@@ -209,6 +212,12 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
 
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     dtype = torch.float32 if args.dtype == "f32" else torch.float64
     index = int(args.config[1])
     wl = make_workload(args.config, dtype, index)

@@ -22,7 +22,7 @@ def randn(shape, seed, dtype=torch.float64):
 
 def rel_err(a, b):
     """max|a-b| / max(1, max|b|): the parity metric of the reference tests (`tests/test_sig.py:88-91`)."""
-    a, b = a.double().cpu(), b.double().cpu()
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
     return float((a - b).abs().max() / max(1.0, float(b.abs().max())))
 
 
