@@ -62,21 +62,25 @@ __device__ __forceinline__ double fmad<double>(double a, double b, double c) { r
 
 // ---------------------------------------------------------------------------------------------
 // one Chen step on a lane's state: chain a[1..P] and sub-trie levels P+1..TOP (TOP <= N)
+//
+// Below the prefix the division by (m - j + 1) is carried by the increment: dxs[q][a] = dx[a] / (q + 1)
+// is staged once per tile, so a sub-trie node is exactly one FMA, tmp_j[w a] = S_j[w a] + tmp_{j-1}[w] * dxs.
+// On the chain (P nodes per target) the parent is scaled instead.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, int P, int M, int J, bool NEG>
 struct StepDescend {
-    // children (level J > P) of a node whose scaled value is ps; idx0 = index of the first child within level J
-    template <int SUB>
-    static __device__ __forceinline__ void run(T ps, int idx0, T (&sub)[SUB], const T (&dx)[D]) {
+    // children (level J > P) of a node with Horner value pt; idx0 = index of the first child within level J
+    template <int SUB, int KS>
+    static __device__ __forceinline__ void run(T pt, int idx0, T (&sub)[SUB], const T (&dxs)[KS][D]) {
         constexpr int off = trie_size(D, J - P - 1);
 #pragma unroll
         for (int a = 0; a < D; ++a) {
-            const T inc = NEG ? -dx[a] : dx[a];
+            const T inc = NEG ? -dxs[M - J][a] : dxs[M - J][a];
             if constexpr (J == M) {
-                sub[off + idx0 + a] = fmad<T>(ps, inc, sub[off + idx0 + a]);
+                sub[off + idx0 + a] = fmad<T>(pt, inc, sub[off + idx0 + a]);
             } else {
-                const T tmp = fmad<T>(ps, inc, sub[off + idx0 + a]);
-                StepDescend<T, D, P, M, J + 1, NEG>::template run<SUB>(tmp * rcp<T>(M - J), (idx0 + a) * D, sub, dx);
+                const T tmp = fmad<T>(pt, inc, sub[off + idx0 + a]);
+                StepDescend<T, D, P, M, J + 1, NEG>::template run<SUB, KS>(tmp, (idx0 + a) * D, sub, dxs);
             }
         }
     }
@@ -84,21 +88,23 @@ struct StepDescend {
 
 template <typename T, int D, int P, int M, bool NEG>
 struct StepTargets {
-    template <int SUB>
-    static __device__ __forceinline__ void run(T (&a)[P + 1], T (&sub)[SUB], const T (&dx)[D], const T (&dxp)[P]) {
+    template <int SUB, int KS>
+    static __device__ __forceinline__ void run(T (&a)[P + 1], T (&sub)[SUB], const T (&dxs)[KS][D],
+                                               const T (&dxp)[P]) {
         T ps = rcp<T>(M);
+        T tmp = T(1);
         constexpr int JP = (M - 1 < P) ? (M - 1) : P;
 #pragma unroll
         for (int j = 1; j <= JP; ++j) {
-            const T tmp = fmad<T>(ps, NEG ? -dxp[j - 1] : dxp[j - 1], a[j]);
+            tmp = fmad<T>(ps, NEG ? -dxp[j - 1] : dxp[j - 1], a[j]);
             ps = tmp * rcp<T>(M - j);
         }
         if constexpr (M <= P) {
             a[M] = fmad<T>(ps, NEG ? -dxp[M - 1] : dxp[M - 1], a[M]);
         } else {
-            StepDescend<T, D, P, M, P + 1, NEG>::template run<SUB>(ps, 0, sub, dx);
+            StepDescend<T, D, P, M, P + 1, NEG>::template run<SUB, KS>(tmp, 0, sub, dxs);
         }
-        if constexpr (M > 1) StepTargets<T, D, P, M - 1, NEG>::template run<SUB>(a, sub, dx, dxp);
+        if constexpr (M > 1) StepTargets<T, D, P, M - 1, NEG>::template run<SUB, KS>(a, sub, dxs, dxp);
     }
 };
 
@@ -107,44 +113,45 @@ struct StepTargets {
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D, int P, int M, int J>
 struct AdjDescend {
-    // returns the adjoint of the scaled parent value ps
-    template <int ASUB, int HSUB>
-    static __device__ __forceinline__ T run(T ps, int idx0, const T (&asub)[ASUB], T (&hsub)[HSUB], const T (&dx)[D],
-                                            T (&gdx)[D]) {
+    // pt = Horner value of the parent; returns its adjoint.  gdxk[q][a] collects the gradient with respect
+    // to dxs[q][a]; the caller folds the 1/(q+1) back in.
+    template <int ASUB, int HSUB, int KS>
+    static __device__ __forceinline__ T run(T pt, int idx0, const T (&asub)[ASUB], T (&hsub)[HSUB],
+                                            const T (&dxs)[KS][D], T (&gdxk)[KS][D]) {
         constexpr int off = trie_size(D, J - P - 1);
-        T gps = T(0);
+        T gpt = T(0);
 #pragma unroll
         for (int a = 0; a < D; ++a) {
             T g;
             if constexpr (J == M) {
                 g = hsub[off + idx0 + a];
             } else {
-                const T tmp = fmad<T>(ps, dx[a], asub[off + idx0 + a]);
-                g = AdjDescend<T, D, P, M, J + 1>::template run<ASUB, HSUB>(tmp * rcp<T>(M - J), (idx0 + a) * D, asub,
-                                                                            hsub, dx, gdx) *
-                    rcp<T>(M - J);
+                const T tmp = fmad<T>(pt, dxs[M - J][a], asub[off + idx0 + a]);
+                g = AdjDescend<T, D, P, M, J + 1>::template run<ASUB, HSUB, KS>(tmp, (idx0 + a) * D, asub, hsub, dxs,
+                                                                                gdxk);
                 hsub[off + idx0 + a] += g;
             }
-            gdx[a] = fmad<T>(g, ps, gdx[a]);
-            gps = fmad<T>(g, dx[a], gps);
+            gdxk[M - J][a] = fmad<T>(g, pt, gdxk[M - J][a]);
+            gpt = fmad<T>(g, dxs[M - J][a], gpt);
         }
-        return gps;
+        return gpt;
     }
 };
 
 template <typename T, int D, int N, int P, int M>
 struct AdjTargets {
     // targets ascending: the seed of target M (adjoint of level M) is only changed by targets above M
-    template <int ASUB, int HSUB>
+    template <int ASUB, int HSUB, int KS>
     static __device__ __forceinline__ void run(const T (&a)[P + 1], const T (&asub)[ASUB], T (&hc)[P + 1],
-                                               T (&hsub)[HSUB], const T (&dx)[D], const T (&dxp)[P], T (&gdx)[D],
-                                               T (&gpre)[P]) {
+                                               T (&hsub)[HSUB], const T (&dxs)[KS][D], const T (&dxp)[P],
+                                               T (&gdxk)[KS][D], T (&gpre)[P]) {
         constexpr int JP = (M - 1 < P) ? (M - 1) : P;
         T ps[P + 2];
+        T tmp = T(1);
         ps[1] = rcp<T>(M);
 #pragma unroll
         for (int j = 1; j <= JP; ++j) {
-            const T tmp = fmad<T>(ps[j], dxp[j - 1], a[j]);
+            tmp = fmad<T>(ps[j], dxp[j - 1], a[j]);
             ps[j + 1] = tmp * rcp<T>(M - j);
         }
         T g;
@@ -152,8 +159,7 @@ struct AdjTargets {
         if constexpr (M <= P) {
             g = hc[M];
         } else {
-            g = AdjDescend<T, D, P, M, P + 1>::template run<ASUB, HSUB>(ps[P + 1], 0, asub, hsub, dx, gdx) *
-                rcp<T>(M - P);
+            g = AdjDescend<T, D, P, M, P + 1>::template run<ASUB, HSUB, KS>(tmp, 0, asub, hsub, dxs, gdxk);
             hc[P] += g;
         }
 #pragma unroll
@@ -164,9 +170,25 @@ struct AdjTargets {
                 hc[j - 1] += g;
             }
         }
-        if constexpr (M < N) AdjTargets<T, D, N, P, M + 1>::template run<ASUB, HSUB>(a, asub, hc, hsub, dx, dxp, gdx, gpre);
+        if constexpr (M < N)
+            AdjTargets<T, D, N, P, M + 1>::template run<ASUB, HSUB, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
     }
 };
+
+// sums over the 16 lanes of a DPP row; every lane of the row ends with the row's sum
+__device__ __forceinline__ float row_total(float v) {
+    v = dpp_add_c<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add_c<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add_c<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add_c<0x140, 0xF>(v);  // row_mirror
+    return v;
+}
+
+__device__ __forceinline__ double row_total(double v) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
 
 struct Span {
     int64_t start, steps;
@@ -191,6 +213,27 @@ __device__ __forceinline__ void chunk_range(int64_t steps, int chunks, int c, in
 }
 
 constexpr int kTile = 64;  // increments staged in LDS at a time
+
+// Stages nt increments as sdx[(tt * KS + q) * D + a] = (x[tt+1][a] - x[tt][a]) / (q + 1).
+template <typename T, int D, int KS, int BLOCK>
+__device__ __forceinline__ void stage_increments(T *sdx, const T *__restrict__ xw, int nt, int tid) {
+    for (int idx = tid; idx < nt * D; idx += BLOCK) {
+        const T inc = xw[idx + D] - xw[idx];
+        const int tt = idx / D, a = idx - tt * D;
+#pragma unroll
+        for (int q = 0; q < KS; ++q) sdx[(tt * KS + q) * D + a] = inc * rcp<T>(q + 1);
+    }
+}
+
+template <typename T, int D, int P, int KS>
+__device__ __forceinline__ void read_increments(const T *sdx, int tt, const int (&u)[P], T (&dxs)[KS][D], T (&dxp)[P]) {
+#pragma unroll
+    for (int q = 0; q < KS; ++q)
+#pragma unroll
+        for (int k = 0; k < D; ++k) dxs[q][k] = sdx[(tt * KS + q) * D + k];
+#pragma unroll
+    for (int j = 0; j < P; ++j) dxp[j] = sdx[tt * KS * D + u[j]];
+}
 
 constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2) : 1; }
 
@@ -375,26 +418,44 @@ __device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], 
 }
 
 // ---------------------------------------------------------------------------------------------
-// forward: one block per unit (row, chunk); writes the unit's signature as a dense-layout row
+// forward: a block holds GW consecutive time chunks of one row, one chunk per group of kBlock threads.
+// Each group sweeps its chunk; the GW chunk signatures are then multiplied together inside the block
+// (pairwise, through LDS), so only one dense-layout row per block goes to memory.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int N, int P>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+template <int D, int N, int P, int GW, typename T>
+constexpr size_t forward_lds_bytes() {
+    using G = Geometry<D, N, P>;
+    return (size_t)GW * kTile * (N - P) * D * sizeof(T) + (size_t)(GW / 2) * G::kSigSize * sizeof(T);
+}
+
+template <typename T, int D, int N, int P, int GW>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
-    __shared__ T sdx[kTile * D];
-    const int pu = threadIdx.x;
+    constexpr int KS = N - P;
+    constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
+    constexpr int kSlotSize = GW > 1 ? (int)G::kSigSize : 4;
+    __shared__ __align__(16) T sdx_all[GW][kTile * KS * D];
+    __shared__ __align__(16) T slot[kSlots][kSlotSize];
+    const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
+    const int pu = (int)threadIdx.x - part * G::kBlock;
+    T *sdx = sdx_all[part];
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
 
-    const int64_t unit = blockIdx.x;
-    const int64_t row = unit / chunks;
-    const int c = (int)(unit - row * chunks);
+    const int groups = chunks / GW;  // blocks per row
+    const int64_t blk = blockIdx.x;
+    const int64_t row = blk / groups;
+    const int c = (int)(blk - row * groups) * GW + part;
     const int64_t b = row / shape.W, w = row - b * shape.W;
     const Span span = unit_span(shape, w);
     int64_t begin, end;
     chunk_range(span.steps, chunks, c, begin, end);
     const T *x = path + (b * shape.L + span.start) * D;
+    // every chunk of the row has floor or ceil of steps/chunks increments: the longest sets the number
+    // of tile rounds for the whole block, so all threads meet at the same barriers
+    const int64_t longest = (span.steps + chunks - 1) / chunks;
 
     T a[P + 1];
     T sub[G::kFwdSub];
@@ -403,22 +464,45 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 #pragma unroll
     for (int i = 0; i < G::kFwdSub; ++i) sub[i] = T(0);
 
-    for (int64_t t0 = begin; t0 < end; t0 += kTile) {
-        const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
+    for (int64_t off = 0; off < longest; off += kTile) {
+        const int64_t t0 = begin + off;
+        const int64_t left = end - t0;
+        const int nt = (int)(left < 0 ? 0 : (left < kTile ? left : kTile));
         const T *xw = x + t0 * D;
         lds_barrier();
-        for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
+        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, pu);
         lds_barrier();
-        for (int tt = 0; tt < nt; ++tt) {
-            T dx[D], dxp[P];
-#pragma unroll
-            for (int k = 0; k < D; ++k) dx[k] = sdx[tt * D + k];
-#pragma unroll
-            for (int j = 0; j < P; ++j) dxp[j] = sdx[tt * D + u[j]];
-            StepTargets<T, D, P, N, false>::template run<G::kFwdSub>(a, sub, dx, dxp);
+        if (nt > 0) {
+            // two register sets of increments: the LDS reads of the next step are issued before the
+            // arithmetic of the current one, so their latency hides behind it
+            T dxs0[KS][D], dxp0[P], dxs1[KS][D], dxp1[P];
+            read_increments<T, D, P, KS>(sdx, 0, u, dxs0, dxp0);
+            int tt = 0;
+            for (; tt + 1 < nt; tt += 2) {
+                read_increments<T, D, P, KS>(sdx, tt + 1, u, dxs1, dxp1);
+                StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
+                read_increments<T, D, P, KS>(sdx, tt + 2 < nt ? tt + 2 : tt + 1, u, dxs0, dxp0);
+                StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs1, dxp1);
+            }
+            if (tt < nt) StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
         }
     }
-    if (active) store_state<T, D, P, N, G::kFwdSub>(out + unit * G::kSigSize, pu, a, sub);
+    if constexpr (GW > 1) {
+        const SubWords<D, P> sw(u);
+#pragma unroll
+        for (int stride = 1; stride < GW; stride *= 2) {
+            const int pair = part / (2 * stride);
+            const bool right = (part % (2 * stride)) == stride;
+            const bool left = (part % (2 * stride)) == 0;
+            lds_barrier();
+            if (right && active) store_state<T, D, P, N, G::kFwdSub>(slot[pair], pu, a, sub);
+            lds_barrier();
+            if (left) apply_right<T, D, P, N, G::kFwdSub>(a, sub, slot[pair], sw);
+        }
+        if (part == 0 && active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
+    } else {
+        if (active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -543,19 +627,46 @@ __device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu,
 // memory during the next round by kCopyThreads extra threads, whose stores nobody waits for.
 constexpr int kCopyThreads = 128;
 
-template <typename T, int COUNT>
-__device__ __forceinline__ void copy_row_out(const T *src_lds, T *__restrict__ dst, int tid) {
-    for (int idx = tid; idx < COUNT; idx += kCopyThreads) dst[idx] = src_lds[idx];
+// Copies one dense-layout row of COUNT elements with THREADS threads, in 16-byte pieces where the row
+// size allows; all loads of a thread are issued before its first store.
+template <typename T, int COUNT, int THREADS>
+__device__ __forceinline__ void copy_row(const T *src, T *dst, int tid) {
+    using Stager = RowStager<T, COUNT, THREADS>;
+    using V = typename Stager::V;
+    const V *s = reinterpret_cast<const V *>(src);
+    V *d = reinterpret_cast<V *>(dst);
+    V regs[Stager::kPer];
+#pragma unroll
+    for (int i = 0; i < Stager::kPer; ++i) {
+        const int idx = i * THREADS + tid;
+        regs[i] = s[idx < Stager::kVecs ? idx : Stager::kVecs - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < Stager::kPer; ++i) {
+        const int idx = i * THREADS + tid;
+        if (idx < Stager::kVecs) d[idx] = regs[i];
+    }
 }
 
-template <typename T, int D, int N, int P>
+template <typename T, int COUNT>
+__device__ __forceinline__ void copy_row_out(const T *src_lds, T *__restrict__ dst, int tid) {
+    copy_row<T, COUNT, kCopyThreads>(src_lds, dst, tid);
+}
+
+// RESIDENT: all chunk rows of the row are first copied into dynamic LDS in one burst (one memory latency
+// for the whole scan); otherwise they stream through a double buffer, one chunk ahead.
+template <typename T, int D, int N, int P, bool RESIDENT>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     dense_scan_kernel(const T *__restrict__ chunk_low, T *__restrict__ edgeA, T *__restrict__ edgeZ, int chunks) {
     using G = Geometry<D, N, P>;
+    using Stager = RowStager<T, (int)G::kLowSize, G::kBlock>;
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
     constexpr int kLow = (int)G::kLowSize;
-    __shared__ __align__(16) T sB[2][RowStager<T, kLow, G::kBlock>::kPadded];
+    constexpr int kThreads = G::kBlock + kCopyThreads;
+    extern __shared__ __align__(16) unsigned char scan_smem[];
+    __shared__ __align__(16) T sB[RESIDENT ? 1 : 2][RESIDENT ? 4 : Stager::kPadded];
     __shared__ __align__(16) T sOut[2][kLow];
+    T *sAll = reinterpret_cast<T *>(scan_smem);  // RESIDENT: [chunks][kLow]
     const bool copier = threadIdx.x >= G::kBlock;
     const int ctid = (int)threadIdx.x - G::kBlock;
     const int pu = copier ? 0 : (int)threadIdx.x;
@@ -565,25 +676,38 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     const SubWords<D, P> sw(u);
     const int64_t row = blockIdx.x;
     const T *rows = chunk_low + row * chunks * kLow;
-    RowStager<T, kLow, G::kBlock> stager;
+    const int last = chunks - 1;
+    if constexpr (RESIDENT) {
+#pragma unroll 8
+        for (int c = 0; c < chunks; ++c)
+            copy_row<T, kLow, kThreads>(rows + (int64_t)c * kLow, sAll + (int64_t)c * kLow, (int)threadIdx.x);
+    }
+    auto chunk_ptr = [&](int c) -> const T * {
+        if constexpr (RESIDENT) return sAll + (int64_t)c * kLow;
+        else return sB[c & 1];
+    };
+    Stager stager;
     T a[P + 1];
     T asub[kAS];
-    const int last = chunks - 1;
     if (blockIdx.y == 0) {
         T *edge = edgeA + row * chunks * kLow;
         if (!copier) {
             load_state<T, D, P, N - 1, kAS>(rows, pu, active, a, asub);
-            stager.fetch(rows + (int64_t)(1 < last ? 1 : last) * kLow);
-            stager.commit(sB[1]);
-            stager.fetch(rows + (int64_t)(2 < last ? 2 : last) * kLow);
+            if constexpr (!RESIDENT) {
+                stager.fetch(rows + (int64_t)(1 < last ? 1 : last) * kLow);
+                stager.commit(sB[1]);
+                stager.fetch(rows + (int64_t)(2 < last ? 2 : last) * kLow);
+            }
             if (active) store_state<T, D, P, N - 1, kAS>(sOut[0], pu, a, asub);
         }
         lds_barrier();
         for (int c = 1; c < chunks; ++c) {
             if (!copier) {
-                apply_right<T, D, P, N - 1, kAS>(a, asub, sB[c & 1], sw);
-                stager.commit(sB[(c + 1) & 1]);
-                stager.fetch(rows + (int64_t)(c + 2 < last ? c + 2 : last) * kLow);
+                apply_right<T, D, P, N - 1, kAS>(a, asub, chunk_ptr(c), sw);
+                if constexpr (!RESIDENT) {
+                    stager.commit(sB[(c + 1) & 1]);
+                    stager.fetch(rows + (int64_t)(c + 2 < last ? c + 2 : last) * kLow);
+                }
                 if (active) store_state<T, D, P, N - 1, kAS>(sOut[c & 1], pu, a, asub);
             } else {
                 copy_row_out<T, kLow>(sOut[(c - 1) & 1], edge + (int64_t)(c - 1) * kLow, ctid);
@@ -596,19 +720,23 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
         // the product to the right of the last chunk is the identity (all coefficients zero)
         if (!copier) {
             for (int idx = threadIdx.x; idx < kLow; idx += G::kBlock) sOut[last & 1][idx] = T(0);
-            stager.fetch(rows + (int64_t)last * kLow);
-            stager.commit(sB[last & 1]);
-            stager.fetch(rows + (int64_t)(last - 1 > 0 ? last - 1 : 0) * kLow);
+            if constexpr (!RESIDENT) {
+                stager.fetch(rows + (int64_t)last * kLow);
+                stager.commit(sB[last & 1]);
+                stager.fetch(rows + (int64_t)(last - 1 > 0 ? last - 1 : 0) * kLow);
+            }
         }
         lds_barrier();
         for (int c = last; c >= 1; --c) {
             if (!copier) {
                 // Z_{c-1} = S_c (x) Z_c
-                load_state<T, D, P, N - 1, kAS>(sB[c & 1], pu, active, a, asub);
+                load_state<T, D, P, N - 1, kAS>(chunk_ptr(c), pu, active, a, asub);
                 apply_right<T, D, P, N - 1, kAS>(a, asub, sOut[c & 1], sw);
                 if (active) store_state<T, D, P, N - 1, kAS>(sOut[(c - 1) & 1], pu, a, asub);
-                stager.commit(sB[(c - 1) & 1]);
-                stager.fetch(rows + (int64_t)(c - 2 > 0 ? c - 2 : 0) * kLow);
+                if constexpr (!RESIDENT) {
+                    stager.commit(sB[(c - 1) & 1]);
+                    stager.fetch(rows + (int64_t)(c - 2 > 0 ? c - 2 : 0) * kLow);
+                }
             } else {
                 copy_row_out<T, kLow>(sOut[c & 1], edge + (int64_t)c * kLow, ctid);
             }
@@ -624,8 +752,12 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                           const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
                           SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
-    __shared__ T sdx[kTile * D];
-    __shared__ T sg[G::kWaves][kTile * D];
+    constexpr int KS = N - P;
+    // per-increment sums leave a wave either as four row sums (when that fits a modest LDS budget) or as
+    // one wave sum; the tile flush adds the parts in a fixed order
+    constexpr int kParts = (G::kWaves * 4 * kTile * D * sizeof(T) <= 16384) ? 4 : 1;
+    __shared__ __align__(16) T sdx[kTile * KS * D];
+    __shared__ T sg[G::kWaves * kParts][kTile * D];
     const int pu = threadIdx.x;
     const int lane = pu & (kWave - 1);
     const int wave = pu / kWave;
@@ -660,6 +792,16 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
         load_state<T, D, P, N - 1, kAS>(sig + row * G::kSigSize, pu, active, a, asub);
     }
     a[0] = T(1);
+    // onehot[j][k] = 1 when the j-th letter of the lane's prefix is k (kept in registers only where
+    // registers are plentiful; otherwise the letters are compared every time)
+    constexpr bool kOneHot = sizeof(T) == 4 && P * D <= 16;
+    T onehot[kOneHot ? P : 1][kOneHot ? D : 1];
+    if constexpr (kOneHot) {
+#pragma unroll
+        for (int j = 0; j < P; ++j)
+#pragma unroll
+            for (int k = 0; k < D; ++k) onehot[j][k] = (u[j] == k) ? T(1) : T(0);
+    }
 
     const int64_t len = end - begin;
     const int64_t ntiles = (len + kTile - 1) / kTile;
@@ -668,37 +810,65 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
         const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
         const T *xw = x + t0 * D;
         lds_barrier();
-        for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) sdx[idx] = xw[idx + D] - xw[idx];
+        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, (int)threadIdx.x);
         lds_barrier();
-        for (int tt = nt - 1; tt >= 0; --tt) {
-            T dx[D], dxp[P];
-#pragma unroll
-            for (int k = 0; k < D; ++k) dx[k] = sdx[tt * D + k];
-#pragma unroll
-            for (int j = 0; j < P; ++j) dxp[j] = sdx[tt * D + u[j]];
+        auto step = [&](int tt, const T (&dxs)[KS][D], const T (&dxp)[P]) {
             // A_t = A_{t+1} (x) exp(-dx_t), levels < N
-            if constexpr (N > 1) StepTargets<T, D, P, N - 1, true>::template run<kAS>(a, asub, dx, dxp);
-            T gdx[D], gpre[P];
+            if constexpr (N > 1) StepTargets<T, D, P, N - 1, true>::template run<kAS, KS>(a, asub, dxs, dxp);
+            T gdxk[KS][D], gpre[P];
 #pragma unroll
-            for (int k = 0; k < D; ++k) gdx[k] = T(0);
+            for (int q = 0; q < KS; ++q)
+#pragma unroll
+                for (int k = 0; k < D; ++k) gdxk[q][k] = T(0);
 #pragma unroll
             for (int j = 0; j < P; ++j) gpre[j] = T(0);
-            AdjTargets<T, D, N, P, 1>::template run<kAS, G::kFwdSub>(a, asub, hc, hsub, dx, dxp, gdx, gpre);
-            // letter k collects the sub-trie sums and the chain positions whose letter is k
+            AdjTargets<T, D, N, P, 1>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
+            // letter k collects the sub-trie sums (with the 1/(q+1) of their increments) and the chain
+            // positions whose letter is k
 #pragma unroll
             for (int k = 0; k < D; ++k) {
-                T v = gdx[k];
+                T v = gdxk[0][k];
 #pragma unroll
-                for (int j = 0; j < P; ++j) v += (u[j] == k) ? gpre[j] : T(0);
-                v = wave_total(v);
-                if (lane == kWave - 1) sg[wave][tt * D + k] = v;
+                for (int q = 1; q < KS; ++q) v = fmad<T>(gdxk[q][k], rcp<T>(q + 1), v);
+#pragma unroll
+                for (int j = 0; j < P; ++j) {
+                    if constexpr (kOneHot) v = fmad<T>(onehot[j][k], gpre[j], v);
+                    else v += (u[j] == k) ? gpre[j] : T(0);
+                }
+                if constexpr (kParts == 4) {
+                    v = row_total(v);
+                    if ((lane & 15) == 0) sg[wave * 4 + (lane >> 4)][tt * D + k] = v;
+                } else {
+                    v = wave_total(v);
+                    if (lane == kWave - 1) sg[wave][tt * D + k] = v;
+                }
+            }
+        };
+        if constexpr (sizeof(T) == 4) {
+            // two register sets of increments, so the LDS reads of the next step hide behind the current one
+            T dxs0[KS][D], dxp0[P], dxs1[KS][D], dxp1[P];
+            int tt = nt - 1;
+            read_increments<T, D, P, KS>(sdx, tt, u, dxs0, dxp0);
+            for (; tt >= 1; tt -= 2) {
+                read_increments<T, D, P, KS>(sdx, tt - 1, u, dxs1, dxp1);
+                step(tt, dxs0, dxp0);
+                read_increments<T, D, P, KS>(sdx, tt - 2 >= 0 ? tt - 2 : 0, u, dxs0, dxp0);
+                step(tt - 1, dxs1, dxp1);
+            }
+            if (tt == 0) step(0, dxs0, dxp0);
+        } else {
+            // fp64 state fills the register file: one set of increments
+            for (int tt = nt - 1; tt >= 0; --tt) {
+                T dxs[KS][D], dxp[P];
+                read_increments<T, D, P, KS>(sdx, tt, u, dxs, dxp);
+                step(tt, dxs, dxp);
             }
         }
         lds_barrier();
         for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
             T v = sg[0][idx];
 #pragma unroll
-            for (int q = 1; q < G::kWaves; ++q) v += sg[q][idx];
+            for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
             if constexpr (ACCUMULATE) {
                 atomicAdd(&ginc[t0 * D + idx], v);
             } else {
@@ -746,8 +916,14 @@ int pick_chunks(int64_t rows, int block, int64_t L) {
     const int64_t max_c = (L - 1) / 16;
     if (c > max_c) c = max_c;
     if (c > 64) c = 64;
+    if (c >= 4) c = (c + 3) / 4 * 4 <= max_c ? (c + 3) / 4 * 4 : c / 4 * 4;  // whole blocks of four chunks
     if (c < 1) c = 1;
     return (int)c;
+}
+
+template <typename T, int D, int N, int P, int GW>
+constexpr bool group_fits() {
+    return Geometry<D, N, P>::kBlock * GW <= 1024 && forward_lds_bytes<D, N, P, GW, T>() <= 64 * 1024;
 }
 
 template <typename T, int D, int N, int P, int PC>
@@ -757,17 +933,34 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
     const int64_t rows = shape.B * shape.W;
     if (chunks <= 1) {
-        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream, path,
-                           sig, shape, 1);
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
+                           path, sig, shape, 1);
         return hipGetLastError();
     }
+    // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits
     T *chunk_sig = (T *)workspace;
-    hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0, stream,
-                       path, chunk_sig, shape, chunks);
+    int groups = chunks;
+    if constexpr (group_fits<T, D, N, P, 4>()) {
+        if (groups == chunks && chunks % 4 == 0) {
+            groups = chunks / 4;
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 4>), dim3((unsigned)(rows * groups)),
+                               dim3(G::kBlock * 4), 0, stream, path, chunk_sig, shape, chunks);
+        }
+    }
+    if constexpr (group_fits<T, D, N, P, 2>()) {
+        if (groups == chunks && chunks % 2 == 0) {
+            groups = chunks / 2;
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 2>), dim3((unsigned)(rows * groups)),
+                               dim3(G::kBlock * 2), 0, stream, path, chunk_sig, shape, chunks);
+        }
+    }
+    if (groups == chunks)
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0,
+                           stream, path, chunk_sig, shape, chunks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, kStaged>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
-                       (const T *)chunk_sig, sig, chunks);
+                       (const T *)chunk_sig, sig, groups);
     return hipGetLastError();
 }
 
@@ -806,12 +999,26 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpH = (T *)ws;
         // chunk signatures below the top level: the depth N-1 forward kernel on the same units
-        hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P>), dim3((unsigned)units),
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P, 1>), dim3((unsigned)units),
                            dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS>), dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), 0, stream,
-                           (const T *)chunk_low, dumpA, dumpH, chunks);
+        // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
+        const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
+        const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
+        if (resident_bytes + fixed_bytes <= 150 * 1024) {
+            auto kernel = dense_scan_kernel<T, D, N, PS, true>;
+            if (resident_bytes > 48 * 1024) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)resident_bytes);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), resident_bytes, stream,
+                               (const T *)chunk_low, dumpA, dumpH, chunks);
+        } else {
+            hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS, false>), dim3((unsigned)rows, 2),
+                               dim3(GC::kBlock + kCopyThreads), 0, stream, (const T *)chunk_low, dumpA, dumpH, chunks);
+        }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         if (accumulate)
