@@ -25,6 +25,9 @@ import time
 import torch
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counters scaled on a
+# copy of known size (summary and commands: profiles/dense_backward_kernel_c2.md)
+TRAFFIC_BYTES = {("c2", "f32"): 50.0e6}
 
 
 # ------------------------------------------------------------------------------------------------
@@ -289,8 +292,28 @@ def main():
         bwd_mean, bwd_med = time_events(lambda: torch.ops.pathsig.signature_backward(*args_b), args.steps, 3)
         ach = 3.0 * wl["fwd_flops"] / (bwd_mean * 1e-3) / 1e12
         result["bwd_ms"] = bwd_med
-        result["roofline"] = {"bound": "valu", "achieved": ach, "peak": peak, "unit": "TFLOP/s", "frac": ach / peak,
-                              "traffic": None, "kernel": "signature backward call"}
+        result["roofline_backward_call"] = {"bound": "valu", "achieved": ach, "peak": peak, "unit": "TFLOP/s",
+                                            "frac": ach / peak, "traffic": None,
+                                            "kernel": "signature backward call (all its launches)"}
+        # the dominant kernel alone: HIP events placed by the library around the reverse-sweep kernel
+        from pathsig_amd import _load
+        lib = _load.lib()
+        lib.pathsig_profile_enable(1)
+        sweep = []
+        for _ in range(args.steps):
+            torch.ops.pathsig.signature_backward(*args_b)
+            ms = float(lib.pathsig_profile_sweep_ms())
+            if ms > 0:
+                sweep.append(ms)
+        lib.pathsig_profile_enable(0)
+        if sweep:
+            sweep_ms = sum(sweep) / len(sweep)
+            ach_k = 3.0 * wl["fwd_flops"] / (sweep_ms * 1e-3) / 1e12
+            result["roofline"] = {"bound": "valu", "achieved": ach_k, "peak": peak, "unit": "TFLOP/s",
+                                  "frac": ach_k / peak, "traffic": TRAFFIC_BYTES.get((args.config, args.dtype)),
+                                  "kernel": "dense_backward_kernel (reverse sweep)", "kernel_ms": sweep_ms}
+        else:
+            result["roofline"] = dict(result["roofline_backward_call"])
     else:
         result["roofline"] = dict(result["roofline_forward"], kernel="signature forward call")
     if not args.no_cpu:

@@ -96,6 +96,16 @@ int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_log
                             int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                             void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Measurement hook (no counterpart in the reference).  While enabled, every backward call that runs the
+ * register-tiled reverse-sweep kernel brackets that one kernel with HIP events on the launch stream.
+ * pathsig_profile_sweep_ms() waits for the events of the last such call and returns the kernel's
+ * duration in milliseconds (a negative value if there was none).  It is the only entry point that
+ * synchronises with the device; the hook is off by default and is not thread safe.
+ */
+int pathsig_profile_enable(int on);
+float pathsig_profile_sweep_ms(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pathsig_last_error.restype = ctypes.c_char_p
     lib.pathsig_last_error.argtypes = []
 
+    lib.pathsig_profile_enable.restype = _INT
+    lib.pathsig_profile_enable.argtypes = [_INT]
+    lib.pathsig_profile_sweep_ms.restype = ctypes.c_float
+    lib.pathsig_profile_sweep_ms.argtypes = []
+
     lib.pathsig_sig_forward_workspace.restype = _SIZE
     lib.pathsig_sig_forward_workspace.argtypes = [_INT, _I64, _I64, _I64, _INT, _PTR, _I64]
     lib.pathsig_sig_forward.restype = _INT

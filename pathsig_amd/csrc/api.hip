@@ -252,6 +252,13 @@ int pathsig_abi_version(void) { return 1; }
 
 const char *pathsig_last_error(void) { return g_error; }
 
+int pathsig_profile_enable(int on) {
+    profile_enable(on != 0);
+    return PATHSIG_OK;
+}
+
+float pathsig_profile_sweep_ms(void) { return profile_sweep_ms(); }
+
 size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
                                      const int64_t *level_sizes, int64_t W) {
     if (check_common(dtype, B, L, d, depth) != PATHSIG_OK) return 0;

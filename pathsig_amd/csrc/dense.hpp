@@ -27,4 +27,8 @@ template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
                                  const DenseChoice &dc, void *workspace, hipStream_t stream);
 
+// measurement hook: events around the reverse-sweep kernel of the last backward call
+void profile_enable(bool on);
+float profile_sweep_ms();
+
 }  // namespace psig

@@ -907,6 +907,20 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 size_t pad256(size_t n) { return (n + 255) / 256 * 256; }
 
+struct SweepProfile {
+    bool enabled = false, valid = false;
+    hipEvent_t start = nullptr, stop = nullptr;
+} g_profile;
+
+void profile_mark(bool begin, hipStream_t stream) {
+    if (!g_profile.enabled) return;
+    if (!g_profile.start) {
+        if (hipEventCreate(&g_profile.start) != hipSuccess || hipEventCreate(&g_profile.stop) != hipSuccess) return;
+    }
+    (void)hipEventRecord(begin ? g_profile.start : g_profile.stop, stream);
+    if (!begin) g_profile.valid = true;
+}
+
 // number of time chunks per row: enough waves to give every SIMD of the GPU about two, but chunks
 // of at least 16 increments
 int pick_chunks(int64_t rows, int block, int64_t L) {
@@ -937,28 +951,29 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            path, sig, shape, 1);
         return hipGetLastError();
     }
-    // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits
+    // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits;
+    // a row that fits one block goes straight to the output, without the combine launch
     T *chunk_sig = (T *)workspace;
     int groups = chunks;
     if constexpr (group_fits<T, D, N, P, 4>()) {
         if (groups == chunks && chunks % 4 == 0) {
             groups = chunks / 4;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 4>), dim3((unsigned)(rows * groups)),
-                               dim3(G::kBlock * 4), 0, stream, path, chunk_sig, shape, chunks);
+                               dim3(G::kBlock * 4), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks);
         }
     }
     if constexpr (group_fits<T, D, N, P, 2>()) {
         if (groups == chunks && chunks % 2 == 0) {
             groups = chunks / 2;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 2>), dim3((unsigned)(rows * groups)),
-                               dim3(G::kBlock * 2), 0, stream, path, chunk_sig, shape, chunks);
+                               dim3(G::kBlock * 2), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks);
         }
     }
     if (groups == chunks)
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0,
                            stream, path, chunk_sig, shape, chunks);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || groups == 1) return e;
     hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, kStaged>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
                        (const T *)chunk_sig, sig, groups);
     return hipGetLastError();
@@ -978,6 +993,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     }
     if (rows == 0) return hipSuccess;
     if (chunks <= 1) {
+        profile_mark(true, stream);
         if (accumulate)
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, false>), dim3((unsigned)rows), dim3(G::kBlock),
                                0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr, grad_inc, shape,
@@ -986,6 +1002,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, false>), dim3((unsigned)rows),
                                dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr,
                                grad_inc, shape, 1);
+        profile_mark(false, stream);
         return hipGetLastError();
     }
     if constexpr (N < 2) {
@@ -1021,6 +1038,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
+        profile_mark(true, stream);
         if (accumulate)
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units), dim3(G::kBlock),
                                0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH, grad_inc, shape,
@@ -1029,11 +1047,25 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
                                dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
                                grad_inc, shape, chunks);
+        profile_mark(false, stream);
         return hipGetLastError();
     }
 }
 
 }  // namespace
+
+void profile_enable(bool on) {
+    g_profile.enabled = on;
+    g_profile.valid = false;
+}
+
+float profile_sweep_ms() {
+    if (!g_profile.valid) return -1.0f;
+    float ms = -1.0f;
+    if (hipEventSynchronize(g_profile.stop) != hipSuccess) return -1.0f;
+    if (hipEventElapsedTime(&ms, g_profile.start, g_profile.stop) != hipSuccess) return -1.0f;
+    return ms;
+}
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,
                          int64_t L, int64_t W, bool) {

@@ -20,7 +20,6 @@ namespace psig {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kLetterLoopMax = 32;  // path dimensions up to this use one wave-wide sum per letter in the backward
 
 template <typename T>
 __device__ __forceinline__ T fma_t(T a, T b, T c);
@@ -124,7 +123,7 @@ __device__ void forward_body(const T *__restrict__ path, T *__restrict__ sig, co
     if (active) sig[row * plan.sig_size + plan.out_off[DEG] + word_idx] = p[DEG];
 }
 
-template <typename T>
+template <typename T, int MAXDEG>
 __global__ void __launch_bounds__(kBlock) words_forward_kernel(const T *__restrict__ path, T *__restrict__ sig,
                                                                SigShape shape, LevelPlan plan,
                                                                const int64_t *__restrict__ codes, int tile) {
@@ -136,8 +135,10 @@ __global__ void __launch_bounds__(kBlock) words_forward_kernel(const T *__restri
     const int deg = find_level(plan, blk);
     const int64_t bl = blk - plan.block_begin[deg];
     switch (deg) {
-#define PSIG_CASE(N) \
-    case N: forward_body<T, N>(path, sig, shape, plan, codes, row, bl, tile, sdx); break;
+#define PSIG_CASE(N)                                                                                  \
+    case N:                                                                                           \
+        if constexpr (N <= MAXDEG) forward_body<T, N>(path, sig, shape, plan, codes, row, bl, tile, sdx); \
+        break;
         PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
         PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
 #undef PSIG_CASE
@@ -145,29 +146,67 @@ __global__ void __launch_bounds__(kBlock) words_forward_kernel(const T *__restri
     }
 }
 
+// The backward runs one wave per block.  For path dimensions up to kSortedMax the per-letter sums of an
+// increment go through a list that is built once per block: the (lane, position) pairs of the wave's
+// words sorted by letter.  Every step each lane drops its per-position gradients into LDS, then adds up
+// DEG consecutive entries of the sorted list (mostly one letter, so mostly one LDS add per lane).
+constexpr int kBwdBlock = kWave;
+constexpr int kSortedMax = 64;
+
 template <typename T, int DEG>
 __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
                               T *__restrict__ grad_inc, const SigShape &shape, const LevelPlan &plan,
                               const int64_t *__restrict__ codes, int64_t row, int64_t blk_in_level, int tile, T *sdx,
-                              T *sacc) {
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
+                              T *sacc, T *sval, int *sorder, int *scnt) {
+    const int lane = threadIdx.x;
     const int64_t d = shape.d;
-    const int64_t word_idx = blk_in_level * kBlock + tid;
+    const int64_t word_idx = blk_in_level * kBwdBlock + lane;
     const bool active = word_idx < plan.size[DEG];
     uint64_t code = 0;
     if (active) code = plan.code_off[DEG] >= 0 ? (uint64_t)codes[plan.code_off[DEG] + word_idx] : (uint64_t)word_idx;
     int l[DEG];
     decode_letters<DEG>(code, (uint64_t)d, l);
+    const bool sorted = d <= kSortedMax;
 
-    // letter positions at which the whole wave holds the same letter are summed across the wave
-    // before they touch LDS
-    unsigned uniform_mask = 0;
+    // entries of the sorted list this lane adds up: source slot in sval, letter
+    int src[DEG], let[DEG];
+    if (sorted) {
+        for (int i = lane; i < (int)d; i += kBwdBlock) scnt[i] = 0;
+        __syncthreads();
+        int pos[DEG];
 #pragma unroll
-    for (int k = 0; k < DEG; ++k) {
-        const int first = __shfl(l[k], 0, kWave);
-        if (__all(l[k] == first)) uniform_mask |= 1u << k;
+        for (int k = 0; k < DEG; ++k) pos[k] = atomicAdd(&scnt[l[k]], 1);
+        __syncthreads();
+        if (lane == 0) {
+            int run = 0;
+            for (int a = 0; a < (int)d; ++a) {
+                const int c = scnt[a];
+                scnt[a] = run;
+                run += c;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < DEG; ++k) sorder[scnt[l[k]] + pos[k]] = (l[k] << 16) | (k * kBwdBlock + lane);
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < DEG; ++e) {
+            const int o = sorder[lane * DEG + e];
+            src[e] = o & 0xffff;
+            let[e] = o >> 16;
+        }
     }
+    // Usual case: the DEG consecutive entries of every lane cover at most two letters.  Then a lane needs
+    // two sums (entries of its first letter, the rest) and at most two LDS adds per step, without branches
+    // inside the entry loop.
+    T first_mask[DEG];
+    int changes = 0;
+#pragma unroll
+    for (int e = 0; e < DEG; ++e) {
+        if (e > 0 && sorted && let[e] != let[e - 1]) ++changes;
+        first_mask[e] = (sorted && let[e] == let[0]) ? T(1) : T(0);
+    }
+    const bool two_runs = sorted && __all(changes <= 1);
 
     const int64_t b = row / shape.W, w = row - b * shape.W;
     const WindowSpan span = window_span(shape, w);
@@ -196,16 +235,14 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
             const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
             const T *xw = x + t0 * d;
             __syncthreads();
-            for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) sdx[idx] = xw[idx + d] - xw[idx];
+            for (int64_t idx = lane; idx < (int64_t)nt * d; idx += kBwdBlock) sdx[idx] = xw[idx + d] - xw[idx];
             __syncthreads();
-            if (active) {
-                for (int tt = 0; tt < nt; ++tt) {
-                    const T *dxr = sdx + (int64_t)tt * d;
-                    T dl[DEG];
+            for (int tt = 0; tt < nt; ++tt) {
+                const T *dxr = sdx + (int64_t)tt * d;
+                T dl[DEG];
 #pragma unroll
-                    for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
-                    chain_step<T, DEG, DEG - 1>(p, dl, T(1));
-                }
+                for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
+                chain_step<T, DEG, DEG - 1>(p, dl, T(1));
             }
         }
     }
@@ -222,89 +259,109 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
         const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
         const T *xw = x + t0 * d;
         __syncthreads();
-        for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) {
+        for (int64_t idx = lane; idx < (int64_t)nt * d; idx += kBwdBlock) {
             sdx[idx] = xw[idx + d] - xw[idx];
             sacc[idx] = T(0);
         }
         __syncthreads();
-        if (active || uniform_mask || d <= kLetterLoopMax) {
-            for (int tt = nt - 1; tt >= 0; --tt) {
-                const T *dxr = sdx + (int64_t)tt * d;
-                T *acc = sacc + (int64_t)tt * d;
-                T dl[DEG];
+        for (int tt = nt - 1; tt >= 0; --tt) {
+            const T *dxr = sdx + (int64_t)tt * d;
+            T *acc = sacc + (int64_t)tt * d;
+            T dl[DEG];
 #pragma unroll
-                for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
-                // S_t = S_{t+1} (x) exp(-dx_t) on the chain (levels < DEG are all the adjoint needs)
-                chain_step<T, DEG, DEG - 1>(p, dl, T(-1));
-                T gl[DEG];
+            for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
+            // S_t = S_{t+1} (x) exp(-dx_t) on the chain (levels < DEG are all the adjoint needs)
+            chain_step<T, DEG, DEG - 1>(p, dl, T(-1));
+            T gl[DEG];
 #pragma unroll
-                for (int k = 0; k < DEG; ++k) gl[k] = T(0);
+            for (int k = 0; k < DEG; ++k) gl[k] = T(0);
 #pragma unroll
-                for (int m = 1; m <= DEG; ++m) {
-                    T s[DEG + 1];
-                    s[1] = Recip<T>::of(m);
+            for (int m = 1; m <= DEG; ++m) {
+                T s[DEG + 1];
+                s[1] = Recip<T>::of(m);
 #pragma unroll
-                    for (int j = 1; j < m; ++j) {
-                        const T tmp = fma_t<T>(s[j], dl[j - 1], p[j]);
-                        s[j + 1] = tmp * Recip<T>::of(m - j);
-                    }
-                    T gt = h[m];
-#pragma unroll
-                    for (int j = m; j >= 1; --j) {
-                        gl[j - 1] = fma_t<T>(gt, s[j], gl[j - 1]);
-                        if (j > 1) {
-                            gt = gt * dl[j - 1] * Recip<T>::of(m - j + 1);
-                            h[j - 1] += gt;
-                        }
-                    }
+                for (int j = 1; j < m; ++j) {
+                    const T tmp = fma_t<T>(s[j], dl[j - 1], p[j]);
+                    s[j + 1] = tmp * Recip<T>::of(m - j);
                 }
-                if (d <= kLetterLoopMax) {
-                    // few letters: one wave-wide sum per letter, then a single lane adds it to the tile
-                    // accumulator (many lanes adding to the same LDS word would serialise badly)
-                    for (int letter = 0; letter < (int)d; ++letter) {
-                        T v = T(0);
+                T gt = h[m];
 #pragma unroll
-                        for (int k = 0; k < DEG; ++k) v += (l[k] == letter) ? gl[k] : T(0);
-                        v = wave_total(v);
-                        if (lane == kWave - 1 && v != T(0)) atomicAdd(&acc[letter], v);
-                    }
-                } else {
-#pragma unroll
-                    for (int k = 0; k < DEG; ++k) {
-                        if (uniform_mask & (1u << k)) {
-                            const T v = wave_sum<T>(gl[k]);
-                            if (lane == 0 && v != T(0)) atomicAdd(&acc[l[k]], v);
-                        } else if (gl[k] != T(0)) {
-                            atomicAdd(&acc[l[k]], gl[k]);
-                        }
+                for (int j = m; j >= 1; --j) {
+                    gl[j - 1] = fma_t<T>(gt, s[j], gl[j - 1]);
+                    if (j > 1) {
+                        gt = gt * dl[j - 1] * Recip<T>::of(m - j + 1);
+                        h[j - 1] += gt;
                     }
                 }
             }
+            if (sorted) {
+                T *val = sval + (tt & 1) * (DEG * kBwdBlock);  // two buffers: one barrier per step is enough
+#pragma unroll
+                for (int k = 0; k < DEG; ++k) val[k * kBwdBlock + lane] = gl[k];
+                __syncthreads();
+                if (two_runs) {
+                    T total = T(0), head = T(0);
+#pragma unroll
+                    for (int e = 0; e < DEG; ++e) {
+                        const T v = val[src[e]];
+                        total += v;
+                        head = fma_t<T>(first_mask[e], v, head);
+                    }
+                    const T tail = total - head;
+                    if (head != T(0)) atomicAdd(&acc[let[0]], head);
+                    if (tail != T(0)) atomicAdd(&acc[let[DEG - 1]], tail);
+                } else {
+                    T run = T(0);
+#pragma unroll
+                    for (int e = 0; e < DEG; ++e) {
+                        run += val[src[e]];
+                        const bool last = (e == DEG - 1) || (let[e + 1 < DEG ? e + 1 : e] != let[e]);
+                        if (last) {
+                            if (run != T(0)) atomicAdd(&acc[let[e]], run);
+                            run = T(0);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < DEG; ++k)
+                    if (gl[k] != T(0)) atomicAdd(&acc[l[k]], gl[k]);
+            }
         }
         __syncthreads();
-        for (int64_t idx = tid; idx < (int64_t)nt * d; idx += kBlock) {
+        for (int64_t idx = lane; idx < (int64_t)nt * d; idx += kBwdBlock) {
             const T v = sacc[idx];
             if (v != T(0)) atomicAdd(&ginc[t0 * d + idx], v);
         }
     }
 }
 
-template <typename T>
-__global__ void __launch_bounds__(kBlock) words_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig,
-                                                                const T *__restrict__ grad_sig, T *__restrict__ grad_inc,
-                                                                SigShape shape, LevelPlan plan,
-                                                                const int64_t *__restrict__ codes, int tile) {
+// MAXDEG bounds the word lengths compiled into one kernel: the register budget of a kernel is that of its
+// longest chain, so shallow signatures get a kernel with more waves per SIMD.
+template <typename T, int MAXDEG>
+__global__ void __launch_bounds__(kBwdBlock) words_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig,
+                                                                   const T *__restrict__ grad_sig,
+                                                                   T *__restrict__ grad_inc, SigShape shape,
+                                                                   LevelPlan plan, const int64_t *__restrict__ codes,
+                                                                   int tile) {
     extern __shared__ __align__(16) unsigned char smem[];
     T *sdx = reinterpret_cast<T *>(smem);
     T *sacc = sdx + (int64_t)tile * shape.d;
+    T *sval = sacc + (int64_t)tile * shape.d;
+    int *sorder = reinterpret_cast<int *>(sval + 2 * plan.depth * kBwdBlock);
+    int *scnt = sorder + plan.depth * kBwdBlock;
     const int64_t per_row = plan.block_begin[plan.depth + 1];
     const int64_t row = (int64_t)blockIdx.x / per_row;
     const int64_t blk = (int64_t)blockIdx.x - row * per_row;
     const int deg = find_level(plan, blk);
     const int64_t bl = blk - plan.block_begin[deg];
     switch (deg) {
-#define PSIG_CASE(N) \
-    case N: backward_body<T, N>(path, sig, grad_sig, grad_inc, shape, plan, codes, row, bl, tile, sdx, sacc); break;
+#define PSIG_CASE(N)                                                                                              \
+    case N:                                                                                                       \
+        if constexpr (N <= MAXDEG)                                                                                \
+            backward_body<T, N>(path, sig, grad_sig, grad_inc, shape, plan, codes, row, bl, tile, sdx, sacc, sval, \
+                                sorder, scnt);                                                                    \
+        break;
         PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
         PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
 #undef PSIG_CASE
@@ -396,9 +453,9 @@ ColumnMap make_column_map(const LevelPlan &plan, int64_t d) {
     return m;
 }
 
-int pick_tile(int64_t d, size_t elem, int64_t max_steps, int arrays) {
-    const int64_t budget = 16384 / arrays;
-    int64_t tile = budget / (int64_t)(d * elem);
+// number of increments staged per tile so that `arrays` LDS arrays of tile * d elements fit `budget` bytes
+int pick_tile(int64_t d, size_t elem, int64_t max_steps, int arrays, int64_t budget) {
+    int64_t tile = budget / arrays / (int64_t)(d * elem);
     if (tile < 1) tile = 1;
     if (tile > 128) tile = 128;
     if (tile > max_steps) tile = max_steps;
@@ -413,23 +470,45 @@ hipError_t launch_words_forward(const T *path, T *sig, const SigShape &shape, co
     const int64_t per_row = plan.block_begin[plan.depth + 1];
     const int64_t blocks = per_row * shape.B * shape.W;
     if (blocks == 0) return hipSuccess;
-    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 1);
+    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 1, 16384);
     const size_t lds = (size_t)tile * shape.d * sizeof(T);
-    hipLaunchKernelGGL(words_forward_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), lds, stream, path, sig, shape,
-                       plan, codes, tile);
+#define PSIG_LAUNCH(MAXDEG)                                                                                    \
+    hipLaunchKernelGGL((words_forward_kernel<T, MAXDEG>), dim3((unsigned)blocks), dim3(kBlock), lds, stream, path, sig, \
+                       shape, plan, codes, tile)
+    if (plan.depth <= 4) PSIG_LAUNCH(4);
+    else if (plan.depth <= 8) PSIG_LAUNCH(8);
+    else PSIG_LAUNCH(12);
+#undef PSIG_LAUNCH
     return hipGetLastError();
 }
 
 template <typename T>
 hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const LevelPlan &plan, const int64_t *codes, hipStream_t stream) {
-    const int64_t per_row = plan.block_begin[plan.depth + 1];
+                                 const LevelPlan &plan_in, const int64_t *codes, hipStream_t stream) {
+    // same levels, blocks of one wave
+    LevelPlan plan = plan_in;
+    int64_t per_row = 0;
+    for (int k = 1; k <= plan.depth; ++k) {
+        plan.block_begin[k] = per_row;
+        per_row += (plan.size[k] + kBwdBlock - 1) / kBwdBlock;
+    }
+    plan.block_begin[plan.depth + 1] = per_row;
     const int64_t blocks = per_row * shape.B * shape.W;
     if (blocks == 0) return hipSuccess;
-    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 2);
-    const size_t lds = (size_t)2 * tile * shape.d * sizeof(T);
-    hipLaunchKernelGGL(words_backward_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), lds, stream, path, sig,
-                       grad_sig, grad_inc, shape, plan, codes, tile);
+    if (blocks >= (int64_t(1) << 31)) return hipErrorInvalidValue;
+    // one wave per block: a small tile keeps many blocks resident on a CU
+    const int tile = pick_tile(shape.d, sizeof(T), shape.L - 1, 2, 4096);
+    const size_t lds = (size_t)2 * tile * shape.d * sizeof(T) + (size_t)2 * plan.depth * kBwdBlock * sizeof(T) +
+                       (size_t)plan.depth * kBwdBlock * sizeof(int) + (size_t)(kSortedMax + 1) * sizeof(int);
+#define PSIG_LAUNCH(MAXDEG)                                                                                       \
+    hipLaunchKernelGGL((words_backward_kernel<T, MAXDEG>), dim3((unsigned)blocks), dim3(kBwdBlock), lds, stream, path, \
+                       sig, grad_sig, grad_inc, shape, plan, codes, tile)
+    if (plan.depth <= 3) PSIG_LAUNCH(3);
+    else if (plan.depth <= 4) PSIG_LAUNCH(4);
+    else if (plan.depth <= 6) PSIG_LAUNCH(6);
+    else if (plan.depth <= 8) PSIG_LAUNCH(8);
+    else PSIG_LAUNCH(12);
+#undef PSIG_LAUNCH
     return hipGetLastError();
 }
 
