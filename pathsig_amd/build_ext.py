@@ -15,7 +15,7 @@ CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB = PKG / "libpathsig_hip.so"
 
-SOURCES = ["api.hip", "words_kernels.hip", "logsig_kernels.hip", "dense_kernels.hip"]
+SOURCES = ["api.hip", "words_kernels.hip", "batch_kernels.hip", "logsig_kernels.hip", "dense_kernels.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -53,6 +53,15 @@ __device__ __forceinline__ float wave_total(float v) {
     return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which on
+// this hardware means waiting for every outstanding global load, including prefetches that are meant to
+// stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ double wave_total(double v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
@@ -72,6 +81,12 @@ hipError_t launch_words_forward(const T *path, T *sig, const SigShape &shape, co
                                 const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
+                                 const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
+// backward with lanes on paths (batch_kernels.hip): same contract as launch_words_backward; usable for
+// batches of at least a dozen paths of moderate dimension
+bool batch_backward_usable(size_t elem, int64_t B, int64_t d, int64_t W);
+template <typename T>
+hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
                                  const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream);

@@ -37,15 +37,6 @@ __device__ __forceinline__ void static_for(F &&f) {
     }
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which on
-// this hardware means waiting for every outstanding global load, including prefetches that are meant to
-// stay in flight across the barrier.
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 constexpr int ipow(int b, int e) { return e <= 0 ? 1 : b * ipow(b, e - 1); }
 // number of sub-trie values in levels 1..k below a prefix
 constexpr int trie_size(int D, int k) { return k <= 0 ? 0 : ipow(D, k) + trie_size(D, k - 1); }

@@ -128,6 +128,73 @@ def test_projection_with_windows(ps):
     assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes, wins)) < 1e-12
 
 
+# Batches of a dozen paths or more take the backward kernels that put lanes on paths (groups of 16 or 32
+# paths per word); the cases cover both group sizes, ragged last groups, dense and listed levels, prefixes
+# read from the saved signature and prefixes rebuilt by a forward sweep, long words and wide alphabets.
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("case", [
+    dict(d=3, depth=4, L=15, B=13, kind="words"),
+    dict(d=3, depth=4, L=40, B=37, kind="gap"),
+    dict(d=5, depth=3, L=23, B=64, kind="dense"),
+    dict(d=16, depth=6, L=19, B=33, kind="c4"),
+    dict(d=2, depth=12, L=9, B=17, kind="long"),
+    dict(d=7, depth=5, L=70, B=24, kind="full_low"),
+    dict(d=40, depth=2, L=11, B=29, kind="dense"),
+    dict(d=3, depth=7, L=12, B=50, kind="dups"),
+])
+def test_projection_backward_lanes_on_paths(ps, dtype, case):
+    d, depth, L, B, kind = case["d"], case["depth"], case["L"], case["B"], case["kind"]
+    if kind == "words":
+        proj = ps.projections.words(random_word_set(d, 1, depth, 45, seed=51), depth=depth, path_dim=d)
+    elif kind == "gap":
+        proj = ps.projections.words([(1,), (0, 1, 2), (2, 2, 1), (1, 0, 0, 2), (1, 0, 0, 2)], depth=depth, path_dim=d)
+    elif kind == "dense":
+        proj = None
+    elif kind == "c4":
+        proj = ps.projections.words(random_word_set(d, 3, 6, 150, seed=52), depth=depth, path_dim=d,
+                                    full_levels=(1, 2))
+    elif kind == "long":
+        proj = ps.projections.words(random_word_set(d, 9, 12, 40, seed=53), depth=depth, path_dim=d,
+                                    full_levels=(1, 2, 3))
+    elif kind == "full_low":
+        proj = ps.projections.words(random_word_set(d, 4, 5, 90, seed=54), depth=depth, path_dim=d,
+                                    full_levels=(1, 2, 3))
+    else:
+        words = random_word_set(d, 2, 7, 30, seed=55)
+        proj = ps.projections.words(sorted(words + words[:9], key=len), depth=depth, path_dim=d)
+    sizes, codes = _plan(proj)
+    path = brownian_path(B, L, d, seed=56) * 1.5
+    big = d ** depth > 200_000  # the level-tensor checker would need the dense top level: per-word checker
+    if big:
+        from oracle import words_oracle as WO
+        want = WO.sig_forward(path, depth, sizes, codes)
+    else:
+        want = TO.compute_signature(path, depth, sizes, codes)
+    G = randn(tuple(want.shape), seed=57)
+    got, grad = _run_sig(ps, path, depth, dtype, projection=proj, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    if big:
+        want_grad = WO.sig_backward(path, want, G, depth, sizes, codes)
+    else:
+        want_grad = TO.signature_vjp(path, G, depth, sizes, codes)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_projection_backward_lanes_on_paths_windows(ps, dtype):
+    d, depth, L, B = 4, 5, 30, 19
+    proj = ps.projections.words(random_word_set(d, 2, 5, 60, seed=61), depth=depth, path_dim=d, full_levels=(1,))
+    wins = [(0, 30), (3, 5), (2, 19), (15, 30), (4, 6), (0, 2), (28, 30), (5, 25), (5, 25), (7, 8), (40, 50)]
+    sizes, codes = _plan(proj)
+    path = brownian_path(B, L, d, seed=62) * 2.0
+    want = TO.compute_signature(path, depth, sizes, codes, wins)
+    G = randn(tuple(want.shape), seed=63)
+    got, grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=wins, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth, sizes, codes, wins)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
 # ------------------------------------------------------------------------------------------------
 # log-signature
 # ------------------------------------------------------------------------------------------------
