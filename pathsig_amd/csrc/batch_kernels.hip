@@ -23,10 +23,11 @@ namespace {
 constexpr int kBatchWaves = 8;
 constexpr int kBatchBlock = kBatchWaves * kWave;
 constexpr int kBatchStride = kWave + 1;
+constexpr int kBatchChunks = 2;  // a tile holds at most kBatchChunks * 64 increments x letters per path
 
 // words swept at once by one lane: chosen so that a wave has about the same work at every word length
 constexpr int batch_words(int deg) {
-    return deg <= 2 ? 8 : deg == 3 ? 6 : deg == 4 ? 4 : deg == 5 ? 3 : deg <= 7 ? 2 : 1;
+    return deg <= 3 ? 8 : deg == 4 ? 6 : deg == 5 ? 4 : deg == 6 ? 3 : deg <= 8 ? 2 : 1;
 }
 
 // level of block `blk` when the levels are laid out from the deepest down: level k owns
@@ -90,33 +91,61 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
         }
     }
 
-    // every wave stages (and later flushes) the paths wave, wave + kBatchWaves, ...: lanes run along time
+    // Every wave stages (and later flushes) the paths wave, wave + kBatchWaves, ...; lanes run along time.
+    // The path points of the next tile are fetched into registers before the current tile is worked on
+    // and turned into increments in LDS after it, so the memory latency hides behind the arithmetic
+    // (the loaded values are first touched in commit()).
     constexpr int kPaths = G / kBatchWaves;
     static_assert(G % kBatchWaves == 0, "paths of a group are dealt out evenly to the waves");
-    auto stage = [&](int64_t t0, int nt) {
+    T fetched_hi[kPaths][kBatchChunks], fetched_lo[kPaths][kBatchChunks];
+    auto fetch = [&](int64_t t0, int nt) {
 #pragma unroll
         for (int pp = 0; pp < kPaths; ++pp) {
             const int q = wave + pp * kBatchWaves;
             const bool ok = b0 + q < shape.B;
             const T *xq = path + ((ok ? b0 + q : 0) * shape.L + span.start + t0) * d;
-            for (int j = lane; j < nt * d; j += kWave) {
-                const T v = ok ? xq[j + d] - xq[j] : T(0);
 #pragma unroll
-                for (int g = 0; g < kSlots; ++g) sdx[j * kStride + g * G + q] = v;
+            for (int c = 0; c < kBatchChunks; ++c) {
+                const int j = lane + c * kWave;
+                const int jc = j < nt * d ? j : 0;
+                fetched_hi[pp][c] = xq[jc + d];
+                fetched_lo[pp][c] = xq[jc];
+            }
+        }
+    };
+    auto commit = [&](int nt) {
+#pragma unroll
+        for (int pp = 0; pp < kPaths; ++pp) {
+            const int q = wave + pp * kBatchWaves;
+            const bool ok = b0 + q < shape.B;
+#pragma unroll
+            for (int c = 0; c < kBatchChunks; ++c) {
+                const int j = lane + c * kWave;
+                if (j < nt * d) {
+                    const T v = ok ? fetched_hi[pp][c] - fetched_lo[pp][c] : T(0);
+#pragma unroll
+                    for (int g = 0; g < kSlots; ++g) sdx[j * kStride + g * G + q] = v;
+                }
             }
         }
     };
     const int slab_size = tile * d * kStride;
     T *slab = slabs + wave * slab_size;
     for (int idx = lane; idx < slab_size; idx += kWave) slab[idx] = T(0);
+    const int64_t ntiles = (span.steps + tile - 1) / tile;
+    auto tile_steps = [&](int64_t ti) {
+        const int64_t left = span.steps - ti * tile;
+        return (int)(left < tile ? left : tile);
+    };
 
-    if (!plan.from_saved[DEG] && DEG > 1) {
+    if (!plan.from_saved[DEG] && DEG > 1 && ntiles > 0) {
         // chain at the right end of the window by a forward sweep (levels < DEG)
-        for (int64_t t0 = 0; t0 < span.steps; t0 += tile) {
-            const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
+        fetch(0, tile_steps(0));
+        commit(tile_steps(0));
+        for (int64_t ti = 0; ti < ntiles; ++ti) {
+            const int nt = tile_steps(ti);
             lds_barrier();
-            stage(t0, nt);
-            lds_barrier();
+            if (ti + 1 < ntiles) fetch((ti + 1) * tile, tile_steps(ti + 1));
             for (int tt = 0; tt < nt; ++tt) {
                 const T *dxr = sdx + tt * d * kStride;
 #pragma unroll
@@ -127,16 +156,21 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
                     chain_step<T, DEG, DEG - 1>(p[i], dl, T(1));
                 }
             }
+            lds_barrier();
+            if (ti + 1 < ntiles) commit(tile_steps(ti + 1));
         }
     }
 
-    const int64_t ntiles = (span.steps + tile - 1) / tile;
+    if (ntiles > 0) {
+        lds_barrier();
+        fetch((ntiles - 1) * tile, tile_steps(ntiles - 1));
+        commit(tile_steps(ntiles - 1));
+    }
     for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
         const int64_t t0 = ti * tile;
-        const int nt = (int)((span.steps - t0) < tile ? (span.steps - t0) : tile);
+        const int nt = tile_steps(ti);
         lds_barrier();
-        stage(t0, nt);
-        lds_barrier();
+        if (ti > 0) fetch((ti - 1) * tile, tile_steps(ti - 1));
         for (int tt = nt - 1; tt >= 0; --tt) {
             const T *dxr = sdx + tt * d * kStride;
             T *acc = slab + tt * d * kStride;
@@ -180,6 +214,7 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
                 if (ok && v != T(0)) atomicAdd(&gq[j], v);
             }
         }
+        if (ti > 0) commit(tile_steps(ti - 1));
     }
 }
 
@@ -231,6 +266,7 @@ int batch_group(int64_t B) {
 
 bool batch_backward_usable(size_t elem, int64_t B, int64_t d, int64_t W) {
     if (B < 12) return false;  // too few paths to fill the lanes: the word-per-lane kernel does better
+    if (d > kBatchChunks * kWave) return false;  // one increment of a path must fit the staging registers
     if (batch_lds_per_step(d, elem) > max_block_lds()) return false;  // one increment of every slab must fit in LDS
     const int64_t groups = (B + 15) / 16;
     return groups * W <= 65535;
@@ -254,6 +290,7 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
     const int64_t per_step = batch_lds_per_step(shape.d, sizeof(T));
     int64_t tile = max_block_lds() / per_step;
     if (tile > 8) tile = 8;
+    if (tile * shape.d > kBatchChunks * kWave) tile = kBatchChunks * kWave / shape.d;
     if (const char *env = getenv("PATHSIG_BATCH_TILE")) {
         const int64_t forced = atoll(env);
         if (forced >= 1 && forced < tile) tile = forced;
