@@ -236,13 +236,9 @@ int check_logsig(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size
     return PATHSIG_OK;
 }
 
-int64_t lower_columns(int64_t d, int depth) {
-    int64_t acc = 0, width = 1;
-    for (int k = 1; k < depth; ++k) {
-        width *= d;
-        acc += width;
-    }
-    return acc;
+size_t logsig_backward_bytes(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
+    const LogsigBackwardPlan lp = logsig_backward_plan(elem_size(dtype), rows, d, depth, top_size);
+    return (size_t)(lp.a_elems + lp.q_elems + lp.top_elems) * elem_size(dtype);
 }
 
 }  // namespace
@@ -352,7 +348,7 @@ int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, in
 
 size_t pathsig_logsig_backward_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
     if (check_logsig(dtype, rows, d, depth, top_size) != PATHSIG_OK) return 0;
-    return align_up((size_t)(rows * lower_columns(d, depth) * depth) * elem_size(dtype)) + 256;
+    return logsig_backward_bytes(dtype, rows, d, depth, top_size) + 256;
 }
 
 int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_logsig, void *grad_sig, int dtype,
@@ -369,7 +365,7 @@ int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_log
         set_error("top_words is NULL but the top level is not dense");
         return PATHSIG_ERR_ARGUMENT;
     }
-    const size_t need = (size_t)(rows * lower_columns(d, depth) * depth) * elem_size(dtype);
+    const size_t need = logsig_backward_bytes(dtype, rows, d, depth, top_size);
     if (need > 0 && (!workspace || workspace_bytes < need)) {
         set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
         return PATHSIG_ERR_WORKSPACE;

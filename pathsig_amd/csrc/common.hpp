@@ -62,9 +62,23 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// the same lane moves for a double: both halves go through the DPP move, then one fp64 add
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_add_c(double v) {
+    const long long bits = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(bits & 0xffffffffll), CTRL, ROW_MASK, 0xF, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(bits >> 32), CTRL, ROW_MASK, 0xF, false);
+    const long long moved = ((long long)hi << 32) | (long long)(unsigned)lo;
+    return v + __builtin_bit_cast(double, moved);
+}
+
 __device__ __forceinline__ double wave_total(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    v = dpp_add_c<0xB1, 0xF>(v);
+    v = dpp_add_c<0x4E, 0xF>(v);
+    v = dpp_add_c<0x141, 0xF>(v);
+    v = dpp_add_c<0x140, 0xF>(v);
+    v = dpp_add_c<0x142, 0xA>(v);
+    v = dpp_add_c<0x143, 0xC>(v);
     return v;
 }
 #endif
@@ -103,9 +117,15 @@ hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B,
 template <typename T>
 hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, int64_t d, int depth, int64_t top_size,
                                  const int64_t *top_words, hipStream_t stream);
+// workspace of the log-signature adjoint, in elements of the floating type (see logsig_kernels.hip)
+struct LogsigBackwardPlan {
+    bool gather;
+    int64_t a_elems, q_elems, top_elems, top_dense;
+};
+LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, int depth, int64_t top_size);
 template <typename T>
-hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *gradP, int64_t rows,
-                                  int64_t d, int depth, int64_t top_size, const int64_t *top_words,
+hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *workspace,
+                                  int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                                   hipStream_t stream);
 
 }  // namespace psig

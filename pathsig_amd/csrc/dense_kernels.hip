@@ -176,8 +176,10 @@ __device__ __forceinline__ float row_total(float v) {
 }
 
 __device__ __forceinline__ double row_total(double v) {
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    v = dpp_add_c<0xB1, 0xF>(v);
+    v = dpp_add_c<0x4E, 0xF>(v);
+    v = dpp_add_c<0x141, 0xF>(v);
+    v = dpp_add_c<0x140, 0xF>(v);
     return v;
 }
 

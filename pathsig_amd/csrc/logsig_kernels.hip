@@ -7,7 +7,16 @@
 //     log S(w) = sum_m (-1)^(m+1)/m * P_m(w).
 // Level n reads the P rows of the levels below it, so levels go up with a workgroup barrier between.
 // Backward (reference: src/pathsig/backward/sig_backward_kernels.cu:381-477) is the adjoint, levels
-// going down; the P adjoint of the lower levels lives in the caller's workspace.
+// going down; the P adjoint of the lower levels lives in the caller's workspace.  Two forms:
+//   * gather form (used whenever a dense copy of the top-level gradient fits the workspace): with
+//     a_m(w) = dL/dP_m(w) and c_m = (-1)^(m+1)/m,
+//         a_m(w) = c_m g(w) + sum_{v, |wv| <= depth} a_{m+1}(wv) S(v),
+//         dL/dS(v) = a_1(v) + sum_{u, |uv| <= depth} sum_{m=2}^{|u|+1} a_m(uv) P_{m-1}(u),
+//     and a_m(x) = c_m g(x) for top-level words x.  Every sum over v (or u) of a fixed length is a
+//     matrix-vector product over a dense level, so each output has one owner and nothing is atomic;
+//   * scatter form (any size): every word pushes its terms to its prefixes and suffixes with atomics.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace psig {
@@ -206,6 +215,151 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
     for (int64_t i = threadIdx.x; i < lds_cols; i += kLogBlock) sink.gs[i] = sink.lds_gs[i];
 }
 
+// ---------------------------------------------------------------------------------------------
+// gather form of the adjoint
+// ---------------------------------------------------------------------------------------------
+// A batch of matrix-vector products by all threads of the block:
+//     out[b][o] = sum_{k < nk} sum_{m < nm} A[b*ab + o*so + k*sk + m*sm] * B[b*bb + k*sb + m*sn]
+// for b < nb, o < no; store(b, o, value) runs once per output, in one thread.  When there are fewer outputs
+// than threads the k range is split over `parts` threads per output and the partial sums meet in LDS
+// (`red`, one element per thread).  Lanes run along whichever of o and k is contiguous in A.  Ends with a
+// block barrier that also orders the stores in global memory for the next call.
+struct MatvecShape {
+    int64_t nb, no, nk, nm;   // batch, outputs, reduction length, inner terms
+    int64_t ab, so, sk, sm;   // strides of A
+    int64_t bb, sb, sn;       // strides of B
+};
+
+template <typename T, typename Store>
+__device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *red, Store &&store) {
+    const int64_t outputs = sh.nb * sh.no;
+    int parts = 1;
+    while ((int64_t)parts * 2 * outputs <= kLogBlock && (int64_t)parts * 2 <= sh.nk) parts *= 2;
+    const int slots = kLogBlock / parts;  // outputs worked on at once; >= outputs whenever parts > 1
+    const bool k_fast = sh.sk < sh.so;
+    const int tid = threadIdx.x;
+    const int part = k_fast ? tid % parts : tid / slots;
+    const int oloc = k_fast ? tid / parts : tid % slots;
+    for (int64_t o0 = 0; o0 < outputs; o0 += slots) {
+        const int64_t oo = o0 + oloc;
+        const int64_t bi = oo / sh.no, o = oo - bi * sh.no;
+        T acc = T(0);
+        if (oo < outputs) {
+            const T *a = A + bi * sh.ab + o * sh.so;
+            const T *bv = B + bi * sh.bb;
+            if (sh.nm == 1) {
+#pragma unroll 16
+                for (int64_t k = part; k < sh.nk; k += parts) acc += a[k * sh.sk] * bv[k * sh.sb];
+            } else {
+                for (int64_t k = part; k < sh.nk; k += parts)
+                    for (int64_t m = 0; m < sh.nm; ++m) acc += a[k * sh.sk + m * sh.sm] * bv[k * sh.sb + m * sh.sn];
+            }
+        }
+        if (parts > 1) {
+            red[tid] = acc;
+            __syncthreads();
+            if (part == 0 && oo < outputs) {
+                T total = T(0);
+                for (int q = 0; q < parts; ++q) total += red[k_fast ? oloc * parts + q : q * slots + oloc];
+                store(bi, o, total);
+            }
+            __syncthreads();
+        } else if (oo < outputs) {
+            store(bi, o, acc);
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+}
+
+// One block per row.  `a` ([lower columns][depth], workspace) holds a_m of the levels below the top, `Q`
+// ([lower columns], workspace) the sums Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) that multiply the top-level
+// gradient, `gtop` the top-level gradient in dense layout (d^depth values per row).
+template <typename T>
+__global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ sig, const T *__restrict__ P,
+                                                                  const T *__restrict__ grad_logsig,
+                                                                  const T *__restrict__ gtop_all, T *grad_sig,
+                                                                  T *a_all, T *Q_all, HybridPlan hp, int64_t top_dense) {
+    __shared__ T red[kLogBlock];
+    const int N = hp.depth;
+    const int64_t row = blockIdx.x;
+    const T *s = sig + row * hp.total;
+    const T *Pr = P + row * hp.total * N;
+    const T *gl = grad_logsig + row * hp.total;
+    const T *gtop = gtop_all + row * top_dense;
+    T *gs = grad_sig + row * hp.total;
+    T *a = a_all + row * hp.lower * N;
+    T *Q = Q_all + row * hp.lower;
+    int64_t width[kMaxDepth + 1];  // d^k
+    width[0] = 1;
+    for (int k = 1; k <= N; ++k) width[k] = width[k - 1] * hp.d;
+
+    // a_m(w) = c_m g(w), Q(w), and zero gradient, for every column below the top; the top-level columns
+    // of the gradient are a_1 = g
+    for (int n = 1; n < N; ++n) {
+        for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
+            const int64_t col = hp.off[n] + i;
+            const T g = gl[col];
+            T q = T(0);
+            for (int m = 1; m <= N; ++m) {
+                a[col * N + m - 1] = m <= n ? alt_coeff<T>(m) * g : T(0);
+                if (m >= 2 && m <= n + 1) q += alt_coeff<T>(m) * Pr[col * N + m - 2];
+            }
+            Q[col] = q;
+            gs[col] = T(0);
+        }
+    }
+    for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) gs[hp.off[N] + i] = gl[hp.off[N] + i];
+    __threadfence_block();
+    __syncthreads();
+
+    // top level: prefix of length j, suffix of length N - j
+    for (int j = 1; j < N; ++j) {
+        const int i = N - j;
+        T *aj = a + hp.off[j] * N;
+        block_matvec<T>(gtop, s + hp.off[i], MatvecShape{1, width[j], width[i], 1, 0, width[i], 1, 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) {
+                            for (int m = 1; m <= j; ++m) aj[o * N + m - 1] += alt_coeff<T>(m + 1) * r;
+                        });
+        T *gsi = gs + hp.off[i];
+        block_matvec<T>(gtop, Q + hp.off[j], MatvecShape{1, width[i], width[j], 1, 0, 1, width[i], 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) { gsi[o] += r; });
+    }
+    // levels below the top, going down: a_m(w) += sum_v a_{m+1}(wv) S(v), all m of a level in one batch
+    for (int n = N - 2; n >= 1; --n) {
+        T *an = a + hp.off[n] * N;
+        for (int i = 1; n + i < N; ++i) {
+            block_matvec<T>(a + hp.off[n + i] * N + 1, s + hp.off[i],
+                            MatvecShape{n, width[n], width[i], 1, 1, width[i] * N, N, 0, 0, 1, 0}, red,
+                            [&](int64_t bi, int64_t o, T r) { an[o * N + bi] += r; });
+        }
+    }
+    // gradient of the lower levels: a_1(v) + sum_u sum_{m=2}^{|u|+1} a_m(uv) P_{m-1}(u)
+    for (int i = 1; i < N; ++i) {
+        T *gsi = gs + hp.off[i];
+        for (int64_t v = threadIdx.x; v < width[i]; v += kLogBlock) gsi[v] += a[(hp.off[i] + v) * N];
+        __threadfence_block();
+        __syncthreads();
+        for (int j = 1; i + j < N; ++j) {
+            block_matvec<T>(a + hp.off[i + j] * N + 1, Pr + hp.off[j] * N,
+                            MatvecShape{1, width[i], width[j], j, 0, N, width[i] * N, 1, 0, N, 1}, red,
+                            [&](int64_t, int64_t o, T r) { gsi[o] += r; });
+        }
+    }
+}
+
+// dense[row][code of word e] += grad_logsig[row][top column e]; dense must be zero on entry
+template <typename T>
+__global__ void scatter_top_kernel(const T *__restrict__ grad_logsig, T *__restrict__ dense, HybridPlan hp,
+                                   const int64_t *__restrict__ top_words, int64_t rows, int64_t top_dense) {
+    const int64_t n = rows * hp.size[hp.depth];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) {
+        const int64_t row = idx / hp.size[hp.depth], e = idx - row * hp.size[hp.depth];
+        atomicAdd(&dense[row * top_dense + top_words[e]], grad_logsig[row * hp.total + hp.off[hp.depth] + e]);
+    }
+}
+
 // largest number of whole low levels whose accumulators (1 + depth values per column) fit `budget` bytes
 int64_t lds_columns(int64_t d, int depth, size_t elem, size_t budget) {
     int64_t cols = 0, width = 1;
@@ -248,12 +402,66 @@ hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, in
     return hipGetLastError();
 }
 
+// Workspace of the adjoint in elements of T: [a: rows x lower x depth][Q: rows x lower][dense top gradient:
+// rows x d^depth, only for a listed top level].  gather = false (scatter form) needs the first part only.
+LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, int depth, int64_t top_size) {
+    LogsigBackwardPlan lp{};
+    int64_t lower = 0, width = 1;
+    for (int k = 1; k < depth; ++k) {
+        width *= d;
+        lower += width;
+    }
+    width *= d;  // d^depth (the caller has checked that it fits)
+    lp.a_elems = rows * lower * depth;
+    lp.q_elems = 0;
+    lp.top_elems = 0;
+    lp.top_dense = width;
+    lp.gather = false;
+    const char *env = getenv("PATHSIG_LOGSIG_SCATTER");
+    const bool forced_scatter = env && env[0] == '1';
+    const bool listed = top_size != width;
+    // the dense copy of the top-level gradient must stay modest: 1 GiB
+    const bool fits = (double)rows * (double)width * (double)elem <= 1073741824.0;
+    if (depth >= 2 && !forced_scatter && (!listed || fits) && rows > 0) {
+        lp.gather = true;
+        lp.q_elems = rows * lower;
+        lp.top_elems = listed ? rows * width : 0;
+    }
+    return lp;
+}
+
 template <typename T>
-hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *gradP, int64_t rows,
-                                  int64_t d, int depth, int64_t top_size, const int64_t *top_words,
+hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *workspace,
+                                  int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                                   hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
     const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
+    const LogsigBackwardPlan lp = logsig_backward_plan(sizeof(T), rows, d, depth, top_size);
+    T *gradP = workspace;
+    if (lp.gather) {
+        T *Q = gradP + lp.a_elems;
+        const T *gtop = grad_logsig + hp.off[depth];
+        int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
+        if (lp.top_elems > 0) {
+            T *dense = Q + lp.q_elems;
+            hipError_t e = launch_fill_zero<T>(dense, lp.top_elems, stream);
+            if (e != hipSuccess) return e;
+            const int64_t n = rows * top_size;
+            if (n > 0) {
+                int64_t blocks = (n + 255) / 256;
+                if (blocks > 65536) blocks = 65536;
+                hipLaunchKernelGGL(scatter_top_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_logsig, dense,
+                                   hp, top_words, rows, lp.top_dense);
+                e = hipGetLastError();
+                if (e != hipSuccess) return e;
+            }
+            gtop = dense;
+            top_stride = lp.top_dense;
+        }
+        hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, P, grad_logsig,
+                           gtop, grad_sig, gradP, Q, hp, top_stride);
+        return hipGetLastError();
+    }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
     const size_t lds_bytes = (size_t)lds_cols * (size_t)(depth + 1) * sizeof(T);
     hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), lds_bytes, stream, sig, P,
