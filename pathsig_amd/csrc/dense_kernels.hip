@@ -183,6 +183,95 @@ __device__ __forceinline__ double row_total(double v) {
     return v;
 }
 
+// Sums of D values (D a power of two, at most 8) over the 16 lanes of a DPP row, all at once: the first
+// log2(D) exchange steps halve the number of values a lane carries (a lane keeps the half selected by one
+// of its index bits and adds its partner's copy of that half), the remaining steps add single values.
+// Exchange partners are lane^1, lane^2, lane^8, lane^4, in that order.  Afterwards every lane holds the
+// row total of letter row_letter<D>(lane); the lanes with row_writer<D>(lane) cover each letter once.
+template <typename T>
+__device__ __forceinline__ T dpp_take_xor4(T v) {
+    // lane^4: banks 0 and 2 of the row read four lanes up, banks 1 and 3 four lanes down
+    if constexpr (sizeof(T) == 4) {
+        int x = __builtin_bit_cast(int, v);
+        int r = __builtin_amdgcn_update_dpp(0, x, 0x104, 0xF, 0x5, false);   // row_shl:4
+        r = __builtin_amdgcn_update_dpp(r, x, 0x114, 0xF, 0xA, false);       // row_shr:4
+        return __builtin_bit_cast(T, r);
+    } else {
+        const long long bits = __builtin_bit_cast(long long, v);
+        const int xl = (int)(bits & 0xffffffffll), xh = (int)(bits >> 32);
+        int rl = __builtin_amdgcn_update_dpp(0, xl, 0x104, 0xF, 0x5, false);
+        rl = __builtin_amdgcn_update_dpp(rl, xl, 0x114, 0xF, 0xA, false);
+        int rh = __builtin_amdgcn_update_dpp(0, xh, 0x104, 0xF, 0x5, false);
+        rh = __builtin_amdgcn_update_dpp(rh, xh, 0x114, 0xF, 0xA, false);
+        return __builtin_bit_cast(T, ((long long)rh << 32) | (long long)(unsigned)rl);
+    }
+}
+
+template <int CTRL, typename T>
+__device__ __forceinline__ T dpp_take(T v) {
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+    } else {
+        const long long bits = __builtin_bit_cast(long long, v);
+        const int lo = __builtin_amdgcn_update_dpp(0, (int)(bits & 0xffffffffll), CTRL, 0xF, 0xF, false);
+        const int hi = __builtin_amdgcn_update_dpp(0, (int)(bits >> 32), CTRL, 0xF, 0xF, false);
+        return __builtin_bit_cast(T, ((long long)hi << 32) | (long long)(unsigned)lo);
+    }
+}
+
+// partner's value for exchange step S (0: lane^1, 1: lane^2, 2: lane^8, 3: lane^4)
+template <int S, typename T>
+__device__ __forceinline__ T row_partner(T v) {
+    if constexpr (S == 0) return dpp_take<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (S == 1) return dpp_take<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (S == 2) return dpp_take<0x128>(v);  // row_ror:8
+    else return dpp_take_xor4(v);
+}
+
+// lane bit that selects the kept half in exchange step S
+__device__ __forceinline__ constexpr int row_step_bit(int S) { return S == 0 ? 1 : S == 1 ? 2 : S == 2 ? 8 : 4; }
+
+template <int D>
+constexpr int log2_of() { return D == 1 ? 0 : 1 + log2_of<D / 2>(); }
+
+template <int D>
+constexpr bool row_transpose_ok() { return D == 2 || D == 4 || D == 8; }
+
+template <int D>
+__device__ __forceinline__ int row_letter(int lane) {
+    int k = 0;
+#pragma unroll
+    for (int s = 0; s < log2_of<D>(); ++s) k += (lane & row_step_bit(s)) ? (D >> (s + 1)) : 0;
+    return k;
+}
+
+template <int D>
+__device__ __forceinline__ bool row_writer(int lane) {
+    bool w = true;
+#pragma unroll
+    for (int s = log2_of<D>(); s < 4; ++s) w = w && !(lane & row_step_bit(s));
+    return w;
+}
+
+template <typename T, int D, int S = 0, int LIVE = D>
+__device__ __forceinline__ T row_totals(T (&v)[D], int lane) {
+    if constexpr (S == 4) {
+        return v[0];
+    } else if constexpr (LIVE > 1) {
+        const bool upper = (lane & row_step_bit(S)) != 0;
+#pragma unroll
+        for (int i = 0; i < LIVE / 2; ++i) {
+            const T keep = upper ? v[i + LIVE / 2] : v[i];
+            const T send = upper ? v[i] : v[i + LIVE / 2];
+            v[i] = keep + row_partner<S>(send);
+        }
+        return row_totals<T, D, S + 1, LIVE / 2>(v, lane);
+    } else {
+        v[0] += row_partner<S>(v[0]);
+        return row_totals<T, D, S + 1, 1>(v, lane);
+    }
+}
+
 struct Span {
     int64_t start, steps;
 };
@@ -746,11 +835,13 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                           SigShape shape, int chunks) {
     using G = Geometry<D, N, P>;
     constexpr int KS = N - P;
-    // per-increment sums leave a wave either as four row sums (when that fits a modest LDS budget) or as
-    // one wave sum; the tile flush adds the parts in a fixed order
-    constexpr int kParts = (G::kWaves * 4 * kTile * D * sizeof(T) <= 16384) ? 4 : 1;
-    __shared__ __align__(16) T sdx[kTile * KS * D];
-    __shared__ T sg[G::kWaves * kParts][kTile * D];
+    // per-increment sums leave a wave as four row sums; the tile flush adds the parts of all waves in a
+    // fixed order.  The tile is shortened until the parts fit 48 KB of LDS.
+    constexpr int kParts = 4;
+    constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
+    constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32 : 16;
+    __shared__ __align__(16) T sdx[kBwdTile * KS * D];
+    __shared__ T sg[G::kWaves * kParts][kBwdTile * D];
     const int pu = threadIdx.x;
     const int lane = pu & (kWave - 1);
     const int wave = pu / kWave;
@@ -787,7 +878,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     a[0] = T(1);
     // onehot[j][k] = 1 when the j-th letter of the lane's prefix is k (kept in registers only where
     // registers are plentiful; otherwise the letters are compared every time)
-    constexpr bool kOneHot = sizeof(T) == 4 && P * D <= 16;
+    constexpr bool kOneHot = sizeof(T) == 4 && P * D <= 24;
     T onehot[kOneHot ? P : 1][kOneHot ? D : 1];
     if constexpr (kOneHot) {
 #pragma unroll
@@ -797,10 +888,10 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     }
 
     const int64_t len = end - begin;
-    const int64_t ntiles = (len + kTile - 1) / kTile;
+    const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
     for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
-        const int64_t t0 = begin + ti * kTile;
-        const int nt = (int)((end - t0) < kTile ? (end - t0) : kTile);
+        const int64_t t0 = begin + ti * kBwdTile;
+        const int nt = (int)((end - t0) < kBwdTile ? (end - t0) : kBwdTile);
         const T *xw = x + t0 * D;
         lds_barrier();
         stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, (int)threadIdx.x);
@@ -818,6 +909,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
             AdjTargets<T, D, N, P, 1>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
             // letter k collects the sub-trie sums (with the 1/(q+1) of their increments) and the chain
             // positions whose letter is k
+            T tot[D];
 #pragma unroll
             for (int k = 0; k < D; ++k) {
                 T v = gdxk[0][k];
@@ -828,12 +920,23 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                     if constexpr (kOneHot) v = fmad<T>(onehot[j][k], gpre[j], v);
                     else v += (u[j] == k) ? gpre[j] : T(0);
                 }
-                if constexpr (kParts == 4) {
-                    v = row_total(v);
-                    if ((lane & 15) == 0) sg[wave * 4 + (lane >> 4)][tt * D + k] = v;
-                } else {
-                    v = wave_total(v);
-                    if (lane == kWave - 1) sg[wave][tt * D + k] = v;
+                tot[k] = v;
+            }
+            if constexpr (kParts == 4 && row_transpose_ok<D>()) {
+                // all letters in one pass of exchanges; one store per row of 16 lanes
+                const T r = row_totals<T, D>(tot, lane);
+                if (row_writer<D>(lane)) sg[wave * 4 + (lane >> 4)][tt * D + row_letter<D>(lane)] = r;
+            } else {
+#pragma unroll
+                for (int k = 0; k < D; ++k) {
+                    T v = tot[k];
+                    if constexpr (kParts == 4) {
+                        v = row_total(v);
+                        if ((lane & 15) == 0) sg[wave * 4 + (lane >> 4)][tt * D + k] = v;
+                    } else {
+                        v = wave_total(v);
+                        if (lane == kWave - 1) sg[wave][tt * D + k] = v;
+                    }
                 }
             }
         };
