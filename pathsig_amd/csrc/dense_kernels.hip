@@ -183,7 +183,7 @@ __device__ __forceinline__ double row_total(double v) {
     return v;
 }
 
-// Sums of D values (D a power of two, at most 8) over the 16 lanes of a DPP row, all at once: the first
+// Sums of D values (D = 2, 4 or 8) over the 16 lanes of a DPP row, all at once: the first
 // log2(D) exchange steps halve the number of values a lane carries (a lane keeps the half selected by one
 // of its index bits and adds its partner's copy of that half), the remaining steps add single values.
 // Exchange partners are lane^1, lane^2, lane^8, lane^4, in that order.  Afterwards every lane holds the
@@ -233,9 +233,6 @@ __device__ __forceinline__ constexpr int row_step_bit(int S) { return S == 0 ? 1
 
 template <int D>
 constexpr int log2_of() { return D == 1 ? 0 : 1 + log2_of<D / 2>(); }
-
-template <int D>
-constexpr bool row_transpose_ok() { return D == 2 || D == 4 || D == 8; }
 
 template <int D>
 __device__ __forceinline__ int row_letter(int lane) {
@@ -922,10 +919,16 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                 }
                 tot[k] = v;
             }
-            if constexpr (kParts == 4 && row_transpose_ok<D>()) {
-                // all letters in one pass of exchanges; one store per row of 16 lanes
-                const T r = row_totals<T, D>(tot, lane);
-                if (row_writer<D>(lane)) sg[wave * 4 + (lane >> 4)][tt * D + row_letter<D>(lane)] = r;
+            if constexpr (kParts == 4 && D <= 8) {
+                // all letters in one pass of exchanges (the alphabet padded to a power of two with zeros);
+                // one store per row of 16 lanes
+                constexpr int DP = D <= 2 ? 2 : D <= 4 ? 4 : 8;
+                T padded[DP];
+#pragma unroll
+                for (int k = 0; k < DP; ++k) padded[k] = k < D ? tot[k] : T(0);
+                const T r = row_totals<T, DP>(padded, lane);
+                const int letter = row_letter<DP>(lane);
+                if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
             } else {
 #pragma unroll
                 for (int k = 0; k < D; ++k) {
