@@ -322,6 +322,81 @@ def test_errors(ps):
     assert ps.Signature(depth=2)(x).shape == (2, 12)
 
 
+# The regimes the reference's own suite sweeps (`tests/test_sig.py:135-152`): depths 7..12, path dimensions
+# up to 100, batches up to 512; and the window / no-projection combinations of LogSignature
+# (`tests/test_windows.py:62-93`).
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,L,B", [
+    (2, 7, 12, 3), (2, 9, 10, 2), (2, 10, 8, 20), (2, 11, 7, 2), (3, 7, 9, 2), (100, 2, 6, 3), (64, 2, 9, 40),
+    (30, 3, 7, 2), (31, 2, 5, 16), (3, 3, 10, 512), (2, 4, 50, 512),
+])
+def test_reference_test_regimes(ps, dtype, d, depth, L, B):
+    path = brownian_path(B, L, d, seed=300 + d + depth) * 1.5
+    want = TO.signature(path, depth)
+    G = randn(tuple(want.shape), seed=301)
+    got, grad = _run_sig(ps, path, depth, dtype, G=G)
+    assert rel_err(got, want) < TOL[dtype]
+    want_grad = TO.signature_vjp(path, G, depth)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", [(3, 4), (2, 6), (8, 2)])
+def test_logsignature_windows_without_projection(ps, dtype, d, depth):
+    B, L = 4, 21
+    wins = [(0, 21), (3, 9), (10, 12), (5, 6), (8, 21)]
+    path = brownian_path(B, L, d, seed=310)
+    want = TO.logsignature(path, depth, wins)
+    G = randn(tuple(want.shape), seed=311)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    win = torch.tensor(wins, dtype=torch.int64, device=DEV)
+    out = ps.LogSignature(depth=depth, windows=win)(x)
+    assert out.shape == want.shape
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    assert rel_err(out.detach(), want) < TOL[dtype]
+    xr = path.clone().requires_grad_(True)
+    (want_grad,) = torch.autograd.grad(TO.logsignature(xr, depth, wins), xr, G)
+    assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
+def test_opcheck_and_compile(ps):
+    """The four ops pass torch's operator checks (schema, fake tensors, autograd registration), as their
+    `pt2_compliant_tag` promises (`bindings.cpp:19`), and the modules trace under torch.compile."""
+    d, depth, B, L = 3, 3, 4, 9
+    x = brownian_path(B, L, d, seed=320).to(DEV)
+    proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    win = torch.tensor([[0, 5], [2, 9]], dtype=torch.int32, device=DEV)
+    empty_w = torch.empty(0, dtype=torch.int64, device=DEV)
+    empty_win = torch.empty((0, 2), dtype=torch.int32, device=DEV)
+    checks = ("test_schema", "test_faketensor", "test_autograd_registration")
+    xg = x.clone().requires_grad_(True)
+    torch.library.opcheck(torch.ops.pathsig.compute_signature.default, (xg, depth, False, empty_w, [], False, empty_win),
+                          test_utils=checks)
+    torch.library.opcheck(torch.ops.pathsig.compute_signature.default,
+                          (xg, depth, True, proj.encoded_words, list(proj.level_sizes), True, win), test_utils=checks)
+    sig = ps.Signature(depth=depth)(x)
+    g = torch.randn_like(sig)
+    torch.library.opcheck(torch.ops.pathsig.signature_backward.default,
+                          (x, sig, g, depth, False, empty_w, [], False, empty_win), test_utils=checks)
+    # the log-signature ops always get the level sizes of the hybrid layout (`modules.py:113-120`)
+    full = [0] + [d ** k for k in range(1, depth + 1)]
+    sg = sig.clone().requires_grad_(True)
+    torch.library.opcheck(torch.ops.pathsig.sig_to_logsig.default, (sg, depth, d, False, empty_w, full), test_utils=checks)
+    logsig, P = torch.ops.pathsig.sig_to_logsig(sig, depth, d, False, empty_w, full)
+    torch.library.opcheck(torch.ops.pathsig.logsig_backward.default,
+                          (sig, P, torch.randn_like(sig), depth, False, empty_w, full), test_utils=checks)
+    mod = ps.LogSignature(depth=depth, projection=proj)
+    compiled = torch.compile(mod, fullgraph=True, backend="aot_eager")
+    xc = x.clone().requires_grad_(True)
+    out = compiled(xc)
+    want = mod(x)
+    assert rel_err(out, want) < 1e-12
+    (gc,) = torch.autograd.grad(out, xc, torch.ones_like(out))
+    xe = x.clone().requires_grad_(True)
+    (ge,) = torch.autograd.grad(mod(xe), xe, torch.ones_like(want))
+    assert rel_err(gc, ge) < 1e-12
+
+
 def test_non_contiguous_and_empty_batch(ps):
     d, depth = 3, 3
     base = brownian_path(2, 8, 2 * d, seed=51)
