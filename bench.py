@@ -311,7 +311,9 @@ def main():
             ach_k = 3.0 * wl["fwd_flops"] / (sweep_ms * 1e-3) / 1e12
             result["roofline"] = {"bound": "valu", "achieved": ach_k, "peak": peak, "unit": "TFLOP/s",
                                   "frac": ach_k / peak, "traffic": TRAFFIC_BYTES.get((args.config, args.dtype)),
-                                  "kernel": "dense_backward_kernel (reverse sweep)", "kernel_ms": sweep_ms}
+                                  "kernel": ("dense_backward_kernel (reverse sweep)" if cfg.get("words") is None
+                                             else "batch_backward_kernel (reverse sweep, lanes on paths)"),
+                                  "kernel_ms": sweep_ms}
         else:
             result["roofline"] = dict(result["roofline_backward_call"])
     else:

@@ -97,8 +97,9 @@ int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_log
                             void *workspace, size_t workspace_bytes, void *stream);
 
 /*
- * Measurement hook (no counterpart in the reference).  While enabled, every backward call that runs the
- * register-tiled reverse-sweep kernel brackets that one kernel with HIP events on the launch stream.
+ * Measurement hook (no counterpart in the reference).  While enabled, every signature backward call brackets
+ * its reverse-sweep kernel (register-tiled, or per-word for general projections) with HIP events on the
+ * launch stream.
  * pathsig_profile_sweep_ms() waits for the events of the last such call and returns the kernel's
  * duration in milliseconds (a negative value if there was none).  It is the only entry point that
  * synchronises with the device; the hook is off by default and is not thread safe.

@@ -198,12 +198,14 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
         e = launch_fill_zero<T>(ginc, B * (L - 1) * d, stream);
         if (e != hipSuccess) return launch_failed(e, "fill launch");
         if (shape.W > 0 && plan.sig_size > 0) {
+            profile_bracket(true, stream);
             if (batch_backward_usable(sizeof(T), B, d, shape.W))
                 e = launch_batch_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan,
                                              codes, stream);
             else
                 e = launch_words_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan,
                                              codes, stream);
+            profile_bracket(false, stream);
             if (e != hipSuccess) return launch_failed(e, "backward launch");
         }
     }

@@ -27,8 +27,10 @@ template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
                                  const DenseChoice &dc, void *workspace, hipStream_t stream);
 
-// measurement hook: events around the reverse-sweep kernel of the last backward call
+// measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
+// the begin and the end of that kernel on its stream; a no-op while the hook is off)
 void profile_enable(bool on);
+void profile_bracket(bool begin, hipStream_t stream);
 float profile_sweep_ms();
 
 }  // namespace psig

@@ -1153,6 +1153,8 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
 
 }  // namespace
 
+void profile_bracket(bool begin, hipStream_t stream) { profile_mark(begin, stream); }
+
 void profile_enable(bool on) {
     g_profile.enabled = on;
     g_profile.valid = false;

@@ -230,8 +230,9 @@ struct MatvecShape {
     int64_t bb, sb, sn;       // strides of B
 };
 
-template <typename T, typename Store>
-__device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *red, Store &&store) {
+// bval(b, k, m) supplies the B operand (strides bb, sb, sn of the shape are not used by this form)
+template <typename T, typename BVal, typename Store>
+__device__ void block_matvec_fn(const T *A, BVal &&bval, const MatvecShape &sh, T *red, Store &&store) {
     const int64_t outputs = sh.nb * sh.no;
     int parts = 1;
     while ((int64_t)parts * 2 * outputs <= kLogBlock && (int64_t)parts * 2 <= sh.nk) parts *= 2;
@@ -246,13 +247,12 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
         T acc = T(0);
         if (oo < outputs) {
             const T *a = A + bi * sh.ab + o * sh.so;
-            const T *bv = B + bi * sh.bb;
             if (sh.nm == 1) {
 #pragma unroll 16
-                for (int64_t k = part; k < sh.nk; k += parts) acc += a[k * sh.sk] * bv[k * sh.sb];
+                for (int64_t k = part; k < sh.nk; k += parts) acc += a[k * sh.sk] * bval(bi, k, (int64_t)0);
             } else {
                 for (int64_t k = part; k < sh.nk; k += parts)
-                    for (int64_t m = 0; m < sh.nm; ++m) acc += a[k * sh.sk + m * sh.sm] * bv[k * sh.sb + m * sh.sn];
+                    for (int64_t m = 0; m < sh.nm; ++m) acc += a[k * sh.sk + m * sh.sm] * bval(bi, k, m);
             }
         }
         if (parts > 1) {
@@ -272,59 +272,98 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
     __syncthreads();
 }
 
-// One block per row.  `a` ([lower columns][depth], workspace) holds a_m of the levels below the top, `Q`
-// ([lower columns], workspace) the sums Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) that multiply the top-level
-// gradient, `gtop` the top-level gradient in dense layout (d^depth values per row).
+template <typename T, typename Store>
+__device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *red, Store &&store) {
+    block_matvec_fn<T>(A, [&](int64_t bi, int64_t k, int64_t m) { return B[bi * sh.bb + k * sh.sb + m * sh.sn]; }, sh, red,
+                       store);
+}
+
+// Top-level part of the gather form, one block per (row, split, side): with the top-level gradient g as a
+// d^j x d^(N-j) matrix, side 0 computes R(u) = sum_v g(uv) S(v) for the prefixes u of length j, side 1
+// computes T(v) = sum_u g(uv) Q(u) for the suffixes v of length N - j, where
+// Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) comes from logsig_q_kernel.  R goes to its own workspace array, T
+// initialises the gradient.
+template <typename T>
+__global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *__restrict__ sig,
+                                                                      const T *__restrict__ Q_all,
+                                                                      const T *__restrict__ gtop_all, T *grad_sig,
+                                                                      T *R_all, HybridPlan hp, int64_t top_dense) {
+    __shared__ T red[kLogBlock];
+    const int N = hp.depth;
+    const int64_t row = blockIdx.x;
+    const int j = (int)blockIdx.y + 1, i = N - j;
+    const bool suffix_side = blockIdx.z == 1;
+    const T *s = sig + row * hp.total;
+    const T *gtop = gtop_all + row * top_dense;
+    int64_t wi = 1, wj = 1;
+    for (int k = 0; k < i; ++k) wi *= hp.d;
+    for (int k = 0; k < j; ++k) wj *= hp.d;
+    if (!suffix_side) {
+        T *R = R_all + row * hp.lower + hp.off[j];
+        block_matvec<T>(gtop, s + hp.off[i], MatvecShape{1, wj, wi, 1, 0, wi, 1, 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) { R[o] = r; });
+    } else {
+        T *gsi = grad_sig + row * hp.total + hp.off[i];
+        block_matvec<T>(gtop, Q_all + row * hp.lower + hp.off[j], MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) { gsi[o] = r; });
+    }
+}
+
+// Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) for every column below the top, all rows
+template <typename T>
+__global__ void logsig_q_kernel(const T *__restrict__ P, T *__restrict__ Q_all, HybridPlan hp, int64_t rows) {
+    const int N = hp.depth;
+    const int64_t total = rows * hp.lower;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t row = idx / hp.lower, col = idx - row * hp.lower;
+        int n = 1;
+        while (n + 1 < N && col >= hp.off[n + 1]) ++n;
+        const T *Pc = P + (row * hp.total + col) * N;
+        T q = T(0);
+        T sign = T(-1);
+        for (int m = 2; m <= n + 1; ++m) {
+            q += sign * Pc[m - 2] / T(m);
+            sign = -sign;
+        }
+        Q_all[idx] = q;
+    }
+}
+
+// Levels below the top, one block per row.  `a` ([lower columns][depth], workspace) holds a_m, `R` ([lower
+// columns], workspace) the top-level sums of logsig_gather_top_kernel, which has also stored the top-level
+// part of the gradient in grad_sig.
 template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ sig, const T *__restrict__ P,
-                                                                  const T *__restrict__ grad_logsig,
-                                                                  const T *__restrict__ gtop_all, T *grad_sig,
-                                                                  T *a_all, T *Q_all, HybridPlan hp, int64_t top_dense) {
+                                                                  const T *__restrict__ grad_logsig, T *grad_sig,
+                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp) {
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
     const int64_t row = blockIdx.x;
     const T *s = sig + row * hp.total;
     const T *Pr = P + row * hp.total * N;
     const T *gl = grad_logsig + row * hp.total;
-    const T *gtop = gtop_all + row * top_dense;
     T *gs = grad_sig + row * hp.total;
     T *a = a_all + row * hp.lower * N;
-    T *Q = Q_all + row * hp.lower;
+    const T *R = R_all + row * hp.lower;
     int64_t width[kMaxDepth + 1];  // d^k
     width[0] = 1;
     for (int k = 1; k <= N; ++k) width[k] = width[k - 1] * hp.d;
 
-    // a_m(w) = c_m g(w), Q(w), and zero gradient, for every column below the top; the top-level columns
-    // of the gradient are a_1 = g
+    // a_m(w) = c_m g(w) + c_{m+1} R(w) for every column below the top; the top-level columns of the
+    // gradient are a_1 = g
     for (int n = 1; n < N; ++n) {
         for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
             const int64_t col = hp.off[n] + i;
-            const T g = gl[col];
-            T q = T(0);
-            for (int m = 1; m <= N; ++m) {
-                a[col * N + m - 1] = m <= n ? alt_coeff<T>(m) * g : T(0);
-                if (m >= 2 && m <= n + 1) q += alt_coeff<T>(m) * Pr[col * N + m - 2];
-            }
-            Q[col] = q;
-            gs[col] = T(0);
+            const T g = gl[col], r = R[col];
+            for (int m = 1; m <= N; ++m)
+                a[col * N + m - 1] = m <= n ? alt_coeff<T>(m) * g + alt_coeff<T>(m + 1) * r : T(0);
         }
     }
     for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) gs[hp.off[N] + i] = gl[hp.off[N] + i];
     __threadfence_block();
     __syncthreads();
 
-    // top level: prefix of length j, suffix of length N - j
-    for (int j = 1; j < N; ++j) {
-        const int i = N - j;
-        T *aj = a + hp.off[j] * N;
-        block_matvec<T>(gtop, s + hp.off[i], MatvecShape{1, width[j], width[i], 1, 0, width[i], 1, 0, 0, 1, 0}, red,
-                        [&](int64_t, int64_t o, T r) {
-                            for (int m = 1; m <= j; ++m) aj[o * N + m - 1] += alt_coeff<T>(m + 1) * r;
-                        });
-        T *gsi = gs + hp.off[i];
-        block_matvec<T>(gtop, Q + hp.off[j], MatvecShape{1, width[i], width[j], 1, 0, 1, width[i], 0, 0, 1, 0}, red,
-                        [&](int64_t, int64_t o, T r) { gsi[o] += r; });
-    }
     // levels below the top, going down: a_m(w) += sum_v a_{m+1}(wv) S(v), all m of a level in one batch
     for (int n = N - 2; n >= 1; --n) {
         T *an = a + hp.off[n] * N;
@@ -402,7 +441,7 @@ hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, in
     return hipGetLastError();
 }
 
-// Workspace of the adjoint in elements of T: [a: rows x lower x depth][Q: rows x lower][dense top gradient:
+// Workspace of the adjoint in elements of T: [a: rows x lower x depth][R, Q: rows x lower each][dense top gradient:
 // rows x d^depth, only for a listed top level].  gather = false (scatter form) needs the first part only.
 LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, int depth, int64_t top_size) {
     LogsigBackwardPlan lp{};
@@ -424,7 +463,7 @@ LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, in
     const bool fits = (double)rows * (double)width * (double)elem <= 1073741824.0;
     if (depth >= 2 && !forced_scatter && (!listed || fits) && rows > 0) {
         lp.gather = true;
-        lp.q_elems = rows * lower;
+        lp.q_elems = 2 * rows * lower;  // R and Q
         lp.top_elems = listed ? rows * width : 0;
     }
     return lp;
@@ -439,11 +478,11 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
     const LogsigBackwardPlan lp = logsig_backward_plan(sizeof(T), rows, d, depth, top_size);
     T *gradP = workspace;
     if (lp.gather) {
-        T *Q = gradP + lp.a_elems;
+        T *R = gradP + lp.a_elems;
         const T *gtop = grad_logsig + hp.off[depth];
         int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
         if (lp.top_elems > 0) {
-            T *dense = Q + lp.q_elems;
+            T *dense = R + lp.q_elems;
             hipError_t e = launch_fill_zero<T>(dense, lp.top_elems, stream);
             if (e != hipSuccess) return e;
             const int64_t n = rows * top_size;
@@ -458,8 +497,19 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
             gtop = dense;
             top_stride = lp.top_dense;
         }
+        T *Q = R + rows * hp.lower;
+        {
+            int64_t blocks = (rows * hp.lower + 255) / 256;
+            if (blocks > 65536) blocks = 65536;
+            if (blocks < 1) blocks = 1;
+            hipLaunchKernelGGL(logsig_q_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, P, Q, hp, rows);
+        }
+        hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2), dim3(kLogBlock), 0,
+                           stream, sig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
         hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, P, grad_logsig,
-                           gtop, grad_sig, gradP, Q, hp, top_stride);
+                           grad_sig, gradP, (const T *)R, hp);
         return hipGetLastError();
     }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
