@@ -234,9 +234,11 @@ def main():
     xg = x.clone().requires_grad_(True)
 
     def step():
+        # forward + backward through autograd; a forward-only workload runs without autograd bookkeeping
+        if not cfg["backward"]:
+            return fwd_only()
         out = mod(xg)
-        if cfg["backward"]:
-            torch.autograd.grad(out, xg, G)
+        torch.autograd.grad(out, xg, G)
 
     # whole-step throughput: W warm-up steps, then exactly K steps between synchronisations
     for _ in range(args.warmup):
