@@ -191,9 +191,11 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
             if (e != hipSuccess) return launch_failed(e, "scatter launch");
             gdense = buf;
         }
+        bool wrote_path = false;
         e = launch_dense_backward<T>((const T *)path, dc.embed ? (const T *)nullptr : (const T *)sig, gdense, ginc,
-                                     shape, dc, extra + dc.dense_bytes, stream);
+                                     (T *)grad_path, &wrote_path, shape, dc, extra + dc.dense_bytes, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
+        if (wrote_path) return PATHSIG_OK;
     } else {
         e = launch_fill_zero<T>(ginc, B * (L - 1) * d, stream);
         if (e != hipSuccess) return launch_failed(e, "fill launch");

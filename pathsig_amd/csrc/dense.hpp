@@ -23,9 +23,12 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
                                 hipStream_t stream);
+// The backward fills grad_inc ([B, L-1, d] increment gradients), or, for time-chunked calls without windows,
+// writes grad_path ([B, L, d]) itself and reports that in *wrote_path.
 template <typename T>
-hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const DenseChoice &dc, void *workspace, hipStream_t stream);
+hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
+                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc, void *workspace,
+                                 hipStream_t stream);
 
 // measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
 // the begin and the end of that kernel on its stream; a no-op while the hook is off)

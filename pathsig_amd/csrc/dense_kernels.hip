@@ -507,9 +507,12 @@ constexpr size_t forward_lds_bytes() {
     return (size_t)GW * kTile * (N - P) * D * sizeof(T) + (size_t)(GW / 2) * G::kSigSize * sizeof(T);
 }
 
+// zero_rows (optional, GW = 1): the block also clears the points of its chunk in a [B, L, D] buffer (the last
+// chunk of a row clears the final point too); the backward uses this to prepare the path gradient.
 template <typename T, int D, int N, int P, int GW>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
-    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks) {
+    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
+                         T *__restrict__ zero_rows = nullptr) {
     using G = Geometry<D, N, P>;
     constexpr int KS = N - P;
     constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
@@ -535,6 +538,13 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
     // every chunk of the row has floor or ceil of steps/chunks increments: the longest sets the number
     // of tile rounds for the whole block, so all threads meet at the same barriers
     const int64_t longest = (span.steps + chunks - 1) / chunks;
+    if constexpr (GW == 1) {
+        if (zero_rows) {
+            const int64_t points = end - begin + (c == chunks - 1 ? 1 : 0);
+            T *z = zero_rows + (b * shape.L + span.start + begin) * D;
+            for (int64_t idx = pu; idx < points * D; idx += G::kBlock) z[idx] = T(0);
+        }
+    }
 
     T a[P + 1];
     T sub[G::kFwdSub];
@@ -829,12 +839,13 @@ template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
                           const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
-                          SigShape shape, int chunks) {
+                          SigShape shape, int chunks, T *__restrict__ grad_path = nullptr) {
     using G = Geometry<D, N, P>;
     constexpr int KS = N - P;
     // per-increment sums leave a wave as four row sums; the tile flush adds the parts of all waves in a
     // fixed order.  The tile is shortened until the parts fit 48 KB of LDS.
     constexpr int kParts = 4;
+    constexpr bool kToPath = CHUNKED && !ACCUMULATE;  // writes the path gradient itself (see the tile flush)
     constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
     constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32 : 16;
     __shared__ __align__(16) T sdx[kBwdTile * KS * D];
@@ -964,14 +975,35 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
             }
         }
         lds_barrier();
-        for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
-            T v = sg[0][idx];
+        if constexpr (kToPath) {
+            // Time-chunked, no windows: the path gradient dL/dx[t] = g[t-1] - g[t] leaves the kernel directly.
+            // Differences inside the tile are stored; the two ends of the tile are added to cells that the
+            // chunk-signature launch has cleared and that receive exactly one more term from the
+            // neighbouring tile (or none at the ends of the path), so the result does not depend on the order.
+            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+                T v = sg[0][idx];
 #pragma unroll
-            for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
-            if constexpr (ACCUMULATE) {
-                atomicAdd(&ginc[t0 * D + idx], v);
-            } else {
-                ginc[t0 * D + idx] = v;
+                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
+                sg[0][idx] = v;
+            }
+            lds_barrier();
+            T *gp = grad_path + (b * shape.L + span.start + t0) * D;
+            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+                const T cur = sg[0][idx];
+                if (idx >= D) gp[idx] = sg[0][idx - D] - cur;
+                else atomicAdd(&gp[idx], -cur);
+                if (idx >= (nt - 1) * D) atomicAdd(&gp[idx + D], cur);
+            }
+        } else {
+            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+                T v = sg[0][idx];
+#pragma unroll
+                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
+                if constexpr (ACCUMULATE) {
+                    atomicAdd(&ginc[t0 * D + idx], v);
+                } else {
+                    ginc[t0 * D + idx] = v;
+                }
             }
         }
     }
@@ -1079,12 +1111,13 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
 }
 
 template <typename T, int D, int N, int P, int PS>
-hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape, int chunks,
-                        void *workspace, hipStream_t stream) {
+hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
+                        const SigShape &shape, int chunks, void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PS>;
     const int64_t rows = shape.B * shape.W;
     const bool accumulate = shape.windows != nullptr;
+    *wrote_path = false;
     hipError_t e;
     if (accumulate) {
         e = launch_fill_zero<T>(grad_inc, shape.B * (shape.L - 1) * shape.d, stream);
@@ -1115,8 +1148,10 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpH = (T *)ws;
         // chunk signatures below the top level: the depth N-1 forward kernel on the same units
+        // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P, 1>), dim3((unsigned)units),
-                           dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks);
+                           dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks,
+                           accumulate ? (T *)nullptr : grad_path);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
@@ -1138,14 +1173,16 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         profile_mark(true, stream);
-        if (accumulate)
+        if (accumulate) {
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units), dim3(G::kBlock),
                                0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH, grad_inc, shape,
-                               chunks);
-        else
+                               chunks, (T *)nullptr);
+        } else {
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
                                dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
-                               grad_inc, shape, chunks);
+                               grad_inc, shape, chunks, grad_path);
+            *wrote_path = true;
+        }
         profile_mark(false, stream);
         return hipGetLastError();
     }
@@ -1209,8 +1246,10 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
 
 #define PSIG_CASE_FWD(I, D, N, P, PC, PS) \
     case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, workspace, stream);
-#define PSIG_CASE_BWD(I, D, N, P, PC, PS) \
-    case I: return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, shape, dc.bwd_chunks, workspace, stream);
+#define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
+    case I:                                                                                                        \
+        return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc.bwd_chunks, \
+                                            workspace, stream);
 
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
@@ -1222,8 +1261,9 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
 }
 
 template <typename T>
-hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const DenseChoice &dc, void *workspace, hipStream_t stream) {
+hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
+                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc, void *workspace,
+                                 hipStream_t stream) {
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_BWD)
         default: return hipErrorNotSupported;
@@ -1233,7 +1273,7 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
 #define PSIG_INSTANTIATE(T)                                                                                    \
     template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const DenseChoice &, void *,  \
                                                 hipStream_t);                                                  \
-    template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, const SigShape &,       \
+    template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, T *, bool *, const SigShape &, \
                                                  const DenseChoice &, void *, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
