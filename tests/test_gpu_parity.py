@@ -412,9 +412,12 @@ def test_long_path_fp32_stays_accurate(ps):
 def test_graph_capture_and_replay(ps):
     """The library only enqueues kernels on the caller's stream (no allocation, no synchronisation, no memset
     nodes), so forward + backward can be captured in a graph; every replay is checked against eager results."""
-    d, depth, B, L = 4, 4, 8, 40
+    d, depth, B, L = 4, 4, 16, 40
     proj = ps.projections.lyndon(depth=depth, path_dim=d)
-    mods = [ps.Signature(depth=depth), ps.LogSignature(depth=depth, projection=proj)]
+    words = ps.projections.words(random_word_set(d, 2, 4, 30, seed=341), depth=depth, path_dim=d, full_levels=(1,))
+    # dense kernels, the log-signature chain, and the per-word kernels (batch of 16: lanes on paths)
+    mods = [ps.Signature(depth=depth), ps.LogSignature(depth=depth, projection=proj),
+            ps.Signature(depth=depth, projection=words)]
     inputs = [brownian_path(B, L, d, seed=340 + i).to(torch.float32).to(DEV) for i in range(3)]
     for mod in mods:
         static_x = inputs[0].clone().requires_grad_(True)
