@@ -115,6 +115,29 @@ def test_projections(ps, dtype, kind):
     assert rel_err(grad, want_grad) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("B", [3, 20])
+def test_anisotropic_projection(ps, dtype, B):
+    """Weighted-degree truncation (`projections.py:132-223`): signature and log-signature through the projection,
+    for a small batch (lanes on words) and a larger one (lanes on paths)."""
+    d, depth, L = 4, 5, 16
+    proj = ps.projections.anisotropic([1.0, 1.5, 2.0, 3.0], weight_threshold=5.0, depth=depth, path_dim=d)
+    assert 0 < proj.sig_size < TO.dense_size(d, depth)
+    sizes, codes = _plan(proj)
+    path = brownian_path(B, L, d, seed=81) * 1.5
+    want = TO.compute_signature(path, depth, sizes, codes)
+    G = randn(tuple(want.shape), seed=82)
+    got, grad = _run_sig(ps, path, depth, dtype, projection=proj, G=G)
+    assert got.shape == (B, proj.sig_size)
+    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes)) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+    # the log-signature in the projection's coordinates equals the gather of the dense log-signature
+    cols = torch.tensor(TO.projection_columns(d, depth, sizes, codes))
+    x = path.to(dtype).to(DEV)
+    out = ps.LogSignature(depth=depth, projection=proj)(x)
+    assert rel_err(out, TO.logsignature(path, depth).index_select(-1, cols)) < TOL[dtype] * 5
+
+
 def test_projection_with_windows(ps):
     d, depth, L, B = 4, 3, 20, 2
     proj = ps.projections.lyndon(depth=depth, path_dim=d)
