@@ -549,6 +549,26 @@ def test_tiled_shapes_time_chunked(ps, monkeypatch, chunks, dtype, d, depth):
     assert rel_err(grad, TO.signature_vjp(path, G, depth)) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
 
 
+@pytest.mark.parametrize("L", [2, 3, 5, 67])
+@pytest.mark.parametrize("d,depth", TILED)
+def test_tiled_shapes_more_chunks_than_increments(ps, monkeypatch, d, depth, L):
+    """Chunks without increments, one-increment chunks, and chunks longer than a tile of the reverse sweep:
+    the backward writes the path gradient chunk by chunk and must leave no point untouched."""
+    monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+    B = 3
+    path = brownian_path(B, L, d, seed=450 + d + depth + L)
+    want = TO.signature(path, depth)
+    G = randn(tuple(want.shape), seed=65)
+    for dtype in (torch.float64, torch.float32):
+        x = path.to(dtype).to(DEV).requires_grad_(True)
+        out = ps.Signature(depth=depth)(x)
+        # a poisoned gradient buffer would show cells that the kernels never write
+        (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+        assert torch.isfinite(grad).all()
+        assert rel_err(out, want) < TOL[dtype]
+        assert rel_err(grad, TO.signature_vjp(path, G, depth)) < TOL[dtype] * (10 if dtype == torch.float32 else 1)
+
+
 @pytest.mark.parametrize("d,depth", [(4, 6), (6, 5)])
 def test_tiled_shapes_time_chunked_windows(ps, monkeypatch, d, depth):
     monkeypatch.setenv("PATHSIG_CHUNKS", "4")
