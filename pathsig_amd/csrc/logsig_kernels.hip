@@ -47,7 +47,8 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *P, T *__restric
     const int depth = hp.depth;
     const uint64_t d = (uint64_t)hp.d;
     const bool listed = (DEG == depth) && hp.top_is_list;
-    for (int64_t i = threadIdx.x; i < hp.size[DEG]; i += kLogBlock) {
+    // the blocks of one row (gridDim.y of them) share the words of the level
+    for (int64_t i = (int64_t)blockIdx.y * kLogBlock + threadIdx.x; i < hp.size[DEG]; i += (int64_t)gridDim.y * kLogBlock) {
         const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
         // dense column of every proper prefix, value of every proper suffix
         uint64_t pidx[DEG + 1];
@@ -85,15 +86,18 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *P, T *__restric
     }
 }
 
+// Levels first..last of one row per blockIdx.x.  Several levels need one block per row (gridDim.y == 1: the
+// barrier between levels is a workgroup barrier); a single level may be shared by gridDim.y blocks.
 template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__restrict__ sig, T *__restrict__ logsig,
                                                                    T *P, HybridPlan hp,
-                                                                   const int64_t *__restrict__ top_words) {
+                                                                   const int64_t *__restrict__ top_words, int first,
+                                                                   int last) {
     const int64_t row = blockIdx.x;
     const T *s = sig + row * hp.total;
     T *lg = logsig + row * hp.total;
     T *Pr = P + row * hp.total * hp.depth;
-    for (int deg = 1; deg <= hp.depth; ++deg) {
+    for (int deg = first; deg <= last; ++deg) {
         switch (deg) {
 #define PSIG_CASE(N) \
     case N: logsig_forward_level<T, N>(s, Pr, lg, hp, top_words); break;
@@ -436,8 +440,21 @@ hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, in
                                  const int64_t *top_words, hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
     const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
+    // The top level only reads the cache rows of the levels below it: when it is large it gets a launch of its
+    // own, with its words dealt out to several blocks per row.
+    int64_t slices = (top_size + 4 * kLogBlock - 1) / (4 * kLogBlock);
+    if (slices > 16) slices = 16;
+    if (depth < 2 || slices < 2) {
+        hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig, P, hp,
+                           top_words, 1, depth);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig, P, hp,
-                       top_words);
+                       top_words, 1, depth - 1);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows, (unsigned)slices), dim3(kLogBlock), 0, stream, sig,
+                       logsig, P, hp, top_words, depth, depth);
     return hipGetLastError();
 }
 
