@@ -644,7 +644,8 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     constexpr int kStage = STAGED ? RowStager<T, (int)G::kSigSize, G::kBlock>::kPadded : 4;
     constexpr int kAhead = 3;
     __shared__ __align__(16) T sB[2][kStage];
-    const int pu = threadIdx.x;
+    // without staging the lanes are independent: the row may then be spread over gridDim.y blocks
+    const int pu = STAGED ? (int)threadIdx.x : (int)(blockIdx.y * blockDim.x + threadIdx.x);
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
@@ -1105,8 +1106,12 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            stream, path, chunk_sig, shape, chunks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || groups == 1) return e;
-    hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, kStaged>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
-                       (const T *)chunk_sig, sig, groups);
+    if constexpr (kStaged)
+        hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, true>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
+                           (const T *)chunk_sig, sig, groups);
+    else
+        hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, false>), dim3((unsigned)rows, (unsigned)GC::kWaves),
+                           dim3(kWave), 0, stream, (const T *)chunk_sig, sig, groups);
     return hipGetLastError();
 }
 
