@@ -26,8 +26,8 @@ import torch
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counters scaled on a
-# copy of known size (summary and commands: profiles/dense_backward_kernel_c2.md)
-TRAFFIC_BYTES = {("c2", "f32"): 50.0e6}
+# copy of known size (summaries and commands: profiles/dense_backward_kernel_c2.md, profiles/dense_kernels_c3_c5.md)
+TRAFFIC_BYTES = {("c2", "f32"): 50.0e6, ("c3", "f32"): 189.7e6, ("c5", "f32"): 57.7e6}
 
 
 # ------------------------------------------------------------------------------------------------
