@@ -42,7 +42,7 @@ def test_c2_full_size_subset_and_properties():
     want = WO.sig_forward(path[:sub], 6)
     assert rel_err(out[:sub], want) < 1e-5
     want_grad = WO.sig_backward(path[:sub], want, G[:sub].double().cpu(), 6)
-    assert rel_err(grad[:sub], want_grad) < 1e-4
+    assert rel_err(grad[:sub], want_grad) < 1e-5
     # Chen: signature of the whole path = product of the signatures of its halves (fp64 on the GPU)
     x64 = path.to(DEV)
     whole = mod(x64)
@@ -80,7 +80,7 @@ def test_c3_windows_full_size():
     sub = 1
     sig_sub = WO.sig_forward(path[:sub], 5, windows=wins)
     want_grad = WO.sig_backward(path[:sub], sig_sub, G[:sub].double().cpu(), 5, windows=wins)
-    assert rel_err(grad[:sub], want_grad) < 1e-4
+    assert rel_err(grad[:sub], want_grad) < 1e-5
     # overlapping windows: gradients add (sum of per-window backward calls == one windowed call), fp64
     x64 = path[:4].to(DEV)
     G64 = G[:4].double()
@@ -108,7 +108,7 @@ def test_c4_word_projection_full_size():
     want = WO.sig_forward(path[:sub], 6, proj.level_sizes, proj._codes)
     assert rel_err(out[:sub], want) < 1e-5
     want_grad = WO.sig_backward(path[:sub], want, G[:sub].double().cpu(), 6, proj.level_sizes, proj._codes)
-    assert rel_err(grad[:sub], want_grad) < 1e-4
+    assert rel_err(grad[:sub], want_grad) < 1e-5
     # levels 1 and 2 are full: they equal the depth-2 dense signature
     import pathsig_amd as ps
     assert rel_err(out[:, :272], ps.Signature(depth=2)(x)) < 1e-5
@@ -132,6 +132,6 @@ def test_c5_logsignature_lyndon_full_size(dtype, tol):
     g_hyb = torch.zeros_like(sig).index_add_(1, idx, G[:sub].double().cpu())
     g_sig = WO.logsig_backward(sig, P, g_hyb, depth, d, top, top_codes)
     want_grad = WO.sig_backward(path[:sub], sig, g_sig, depth, mod._ext_level_sizes, top_codes)
-    assert rel_err(grad[:sub], want_grad) < tol * 10
+    assert rel_err(grad[:sub], want_grad) < tol
     # level 1 of a log-signature is the total increment
     assert rel_err(out[:, :8], (path[:, -1] - path[:, 0])) < tol
