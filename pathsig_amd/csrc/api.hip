@@ -144,7 +144,9 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
         // a dense call writes straight into sig; an embedded projection goes through a dense buffer
         T *dense = dc.embed ? (T *)workspace : (T *)sig;
         void *rest = (unsigned char *)workspace + dc.dense_bytes;
-        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, rest, stream);
+        const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
+        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, top_codes, plan.size[depth], rest,
+                                               stream);
         if (e != hipSuccess) return launch_failed(e, "dense forward launch");
         if (dc.embed) {
             e = launch_gather_columns<T>(dense, (T *)sig, plan, d, codes, B * shape.W, stream);
@@ -192,8 +194,10 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
             gdense = buf;
         }
         bool wrote_path = false;
+        const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
         e = launch_dense_backward<T>((const T *)path, dc.embed ? (const T *)nullptr : (const T *)sig, gdense, ginc,
-                                     (T *)grad_path, &wrote_path, shape, dc, extra + dc.dense_bytes, stream);
+                                     (T *)grad_path, &wrote_path, shape, dc, top_codes, plan.size[depth],
+                                     extra + dc.dense_bytes, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
         if (wrote_path) return PATHSIG_OK;
     } else {

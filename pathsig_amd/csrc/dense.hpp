@@ -8,6 +8,7 @@ namespace psig {
 struct DenseChoice {
     bool usable;                // a register-tiled kernel exists for this call
     bool embed;                 // the call is a word projection that is computed densely and then gathered
+    bool bounded;               // embed: the sweeps leave out top-level words by the letter bounds of the word list
     int variant;                // index into the table of compiled shapes
     int fwd_chunks;             // time chunks per (path, window) in the forward
     int bwd_chunks;             // ... and in the backward (at least 2 when embedding: no dense signature is saved)
@@ -20,15 +21,16 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
                          int64_t L, int64_t W, bool windowed);
 
 // `sig` / `grad_sig` are dense-layout rows; `workspace` is the part of the scratch after any dense buffer.
+// top_codes / top_count: the word list of the top level (device memory), read only when dc.bounded.
 template <typename T>
-hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
-                                hipStream_t stream);
+hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
+                                const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream);
 // The backward fills grad_inc ([B, L-1, d] increment gradients), or, for time-chunked calls without windows,
 // writes grad_path ([B, L, d]) itself and reports that in *wrote_path.
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
-                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc, void *workspace,
-                                 hipStream_t stream);
+                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
+                                 const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream);
 
 // measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
 // the begin and the end of that kernel on its stream; a no-op while the hook is off)

@@ -19,6 +19,7 @@
 // step (which yields H_{t-1} and dL/d(dx_t)), and keeps the top level of H equal to the upstream
 // gradient.  Adjoint values of the shared chain nodes stay lane-private partial sums (everything they
 // feed is linear in them), so the only cross-lane operation is the final sum of D numbers per step.
+#include <cmath>
 #include <cstdlib>
 #include <type_traits>
 
@@ -34,6 +35,17 @@ __device__ __forceinline__ void static_for(F &&f) {
     if constexpr (Begin < End) {
         f(std::integral_constant<int, Begin>{});
         static_for<Begin + 1, End>(f);
+    }
+}
+
+// f(std::integral_constant<int, v>) for the one v in [Begin, End] equal to `value` (End when none below it is)
+template <int Begin, int End, typename F>
+__device__ __forceinline__ void dispatch_value(int value, F &&f) {
+    if constexpr (Begin >= End) {
+        f(std::integral_constant<int, End>{});
+    } else {
+        if (value == Begin) f(std::integral_constant<int, Begin>{});
+        else dispatch_value<Begin + 1, End>(value, f);
     }
 }
 
@@ -58,26 +70,28 @@ __device__ __forceinline__ double fmad<double>(double a, double b, double c) { r
 // is staged once per tile, so a sub-trie node is exactly one FMA, tmp_j[w a] = S_j[w a] + tmp_{j-1}[w] * dxs.
 // On the chain (P nodes per target) the parent is scaled instead.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int P, int M, int J, bool NEG>
+// LO: letters below LO are left out below the prefix (their words are not wanted; see LetterBounds).
+template <typename T, int D, int P, int M, int J, bool NEG, int LO = 0>
 struct StepDescend {
     // children (level J > P) of a node with Horner value pt; idx0 = index of the first child within level J
     template <int SUB, int KS>
     static __device__ __forceinline__ void run(T pt, int idx0, T (&sub)[SUB], const T (&dxs)[KS][D]) {
         constexpr int off = trie_size(D, J - P - 1);
 #pragma unroll
-        for (int a = 0; a < D; ++a) {
+        for (int a = LO; a < D; ++a) {
             const T inc = NEG ? -dxs[M - J][a] : dxs[M - J][a];
             if constexpr (J == M) {
                 sub[off + idx0 + a] = fmad<T>(pt, inc, sub[off + idx0 + a]);
             } else {
                 const T tmp = fmad<T>(pt, inc, sub[off + idx0 + a]);
-                StepDescend<T, D, P, M, J + 1, NEG>::template run<SUB, KS>(tmp, (idx0 + a) * D, sub, dxs);
+                StepDescend<T, D, P, M, J + 1, NEG, LO>::template run<SUB, KS>(tmp, (idx0 + a) * D, sub, dxs);
             }
         }
     }
 };
 
-template <typename T, int D, int P, int M, bool NEG>
+// LO applies to the top target only (the first M of the recursion); the targets below are complete.
+template <typename T, int D, int P, int M, bool NEG, int LO = 0>
 struct StepTargets {
     template <int SUB, int KS>
     static __device__ __forceinline__ void run(T (&a)[P + 1], T (&sub)[SUB], const T (&dxs)[KS][D],
@@ -93,7 +107,7 @@ struct StepTargets {
         if constexpr (M <= P) {
             a[M] = fmad<T>(ps, NEG ? -dxp[M - 1] : dxp[M - 1], a[M]);
         } else {
-            StepDescend<T, D, P, M, P + 1, NEG>::template run<SUB, KS>(tmp, 0, sub, dxs);
+            StepDescend<T, D, P, M, P + 1, NEG, LO>::template run<SUB, KS>(tmp, 0, sub, dxs);
         }
         if constexpr (M > 1) StepTargets<T, D, P, M - 1, NEG>::template run<SUB, KS>(a, sub, dxs, dxp);
     }
@@ -102,7 +116,7 @@ struct StepTargets {
 // ---------------------------------------------------------------------------------------------
 // adjoint of one Chen step
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int P, int M, int J>
+template <typename T, int D, int P, int M, int J, int LO = 0>
 struct AdjDescend {
     // pt = Horner value of the parent; returns its adjoint.  gdxk[q][a] collects the gradient with respect
     // to dxs[q][a]; the caller folds the 1/(q+1) back in.
@@ -112,14 +126,14 @@ struct AdjDescend {
         constexpr int off = trie_size(D, J - P - 1);
         T gpt = T(0);
 #pragma unroll
-        for (int a = 0; a < D; ++a) {
+        for (int a = LO; a < D; ++a) {
             T g;
             if constexpr (J == M) {
                 g = hsub[off + idx0 + a];
             } else {
                 const T tmp = fmad<T>(pt, dxs[M - J][a], asub[off + idx0 + a]);
-                g = AdjDescend<T, D, P, M, J + 1>::template run<ASUB, HSUB, KS>(tmp, (idx0 + a) * D, asub, hsub, dxs,
-                                                                                gdxk);
+                g = AdjDescend<T, D, P, M, J + 1, LO>::template run<ASUB, HSUB, KS>(tmp, (idx0 + a) * D, asub, hsub,
+                                                                                    dxs, gdxk);
                 hsub[off + idx0 + a] += g;
             }
             gdxk[M - J][a] = fmad<T>(g, pt, gdxk[M - J][a]);
@@ -129,9 +143,10 @@ struct AdjDescend {
     }
 };
 
-template <typename T, int D, int N, int P, int M>
+template <typename T, int D, int N, int P, int M, int LO = 0>
 struct AdjTargets {
-    // targets ascending: the seed of target M (adjoint of level M) is only changed by targets above M
+    // targets ascending: the seed of target M (adjoint of level M) is only changed by targets above M;
+    // LO applies to the top target (M = N), whose left-out words have a zero upstream gradient
     template <int ASUB, int HSUB, int KS>
     static __device__ __forceinline__ void run(const T (&a)[P + 1], const T (&asub)[ASUB], T (&hc)[P + 1],
                                                T (&hsub)[HSUB], const T (&dxs)[KS][D], const T (&dxp)[P],
@@ -150,7 +165,8 @@ struct AdjTargets {
         if constexpr (M <= P) {
             g = hc[M];
         } else {
-            g = AdjDescend<T, D, P, M, P + 1>::template run<ASUB, HSUB, KS>(tmp, 0, asub, hsub, dxs, gdxk);
+            g = AdjDescend<T, D, P, M, P + 1, (M == N ? LO : 0)>::template run<ASUB, HSUB, KS>(tmp, 0, asub, hsub, dxs,
+                                                                                                 gdxk);
             hc[P] += g;
         }
 #pragma unroll
@@ -162,7 +178,7 @@ struct AdjTargets {
             }
         }
         if constexpr (M < N)
-            AdjTargets<T, D, N, P, M + 1>::template run<ASUB, HSUB, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
+            AdjTargets<T, D, N, P, M + 1, LO>::template run<ASUB, HSUB, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
     }
 };
 
@@ -267,6 +283,59 @@ __device__ __forceinline__ T row_totals(T (&v)[D], int lane) {
         v[0] += row_partner<S>(v[0]);
         return row_totals<T, D, S + 1, 1>(v, lane);
     }
+}
+
+// Letter bounds of a set of top-level words: bounds[a] = the smallest letter that occurs after the first
+// letter in any wanted word that starts with a (D when no word starts with a).  A word a w_2 .. w_N with
+// some w_j < bounds[a] is therefore not wanted, and the sweeps leave its sub-trie node out.  The bound has
+// to be the same for all lanes of a wave, which holds when the lanes of a wave share their first letter.
+template <int D, int P>
+struct LetterBounds {
+    static constexpr int kPerLetter = ipow(D, P - 1);  // lanes that share a first letter
+    static constexpr bool kUsable = P >= 1 && kPerLetter % kWave == 0;
+    static __device__ __forceinline__ int of_wave(const int *__restrict__ bounds, int pu) {
+        const int first = __builtin_amdgcn_readfirstlane(pu / kPerLetter);
+        const int lo = bounds[first];
+        return lo < 0 ? 0 : (lo > D ? D : lo);
+    }
+    // Prefix of thread tid.  The first letters are dealt to the waves in the order 0, 1, .., D/2-1, D-1, .., D/2:
+    // bounds tend to grow with the first letter (Lyndon words), and waves that are four apart tend to share a
+    // SIMD, so this pairs a long sweep with a short one.
+    static __device__ __forceinline__ int prefix_of_thread(int tid) {
+        const int first = tid / kPerLetter;
+        const int dealt = first < D / 2 ? first : D - 1 - (first - D / 2);
+        return dealt * kPerLetter + (tid - first * kPerLetter);
+    }
+};
+
+// bounds[0..d) from the codes of the top-level words (one block; d <= 16)
+template <typename C>
+__device__ __forceinline__ void least_later_letter(C c, C d, int depth, int &first, int &least) {
+    least = (int)d;
+    for (int j = 1; j < depth; ++j) {
+        const C q = c / d;
+        const int letter = (int)(c - q * d);
+        c = q;
+        least = letter < least ? letter : least;
+    }
+    first = (int)(c % d);
+}
+
+__global__ void __launch_bounds__(1024)
+    letter_bounds_kernel(const int64_t *__restrict__ codes, int64_t count, int d, int depth, bool narrow,
+                         int *__restrict__ bounds) {
+    __shared__ int lo[16];
+    if (threadIdx.x < 16) lo[threadIdx.x] = d;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < count; i += blockDim.x) {
+        int first, least;
+        // codes below 2^32 are taken apart with 32-bit divisions
+        if (narrow) least_later_letter<uint32_t>((uint32_t)codes[i], (uint32_t)d, depth, first, least);
+        else least_later_letter<uint64_t>((uint64_t)codes[i], (uint64_t)d, depth, first, least);
+        if (least < lo[first]) atomicMin(&lo[first], least);
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < d) bounds[threadIdx.x] = lo[threadIdx.x];
 }
 
 struct Span {
@@ -509,18 +578,27 @@ constexpr size_t forward_lds_bytes() {
 
 // zero_rows (optional, GW = 1): the block also clears the points of its chunk in a [B, L, D] buffer (the last
 // chunk of a row clears the final point too); the backward uses this to prepare the path gradient.
+// BOUND: top-level words with a letter below BOUND after the prefix's first letter are left out (they stay zero
+// in the output); the LDS arrays belong to the calling kernel.
 template <typename T, int D, int N, int P, int GW>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
-    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
-                         T *__restrict__ zero_rows = nullptr) {
+struct ForwardShape {
+    using G = Geometry<D, N, P>;
+    static constexpr int KS = N - P;
+    static constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
+    static constexpr int kSlotSize = GW > 1 ? (int)G::kSigSize : 4;
+    static constexpr int kStage = kTile * KS * D;  // staged increments of one chunk
+};
+
+template <typename T, int D, int N, int P, int GW, int BOUND>
+__device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T *__restrict__ out,
+                                                   const SigShape &shape, int chunks, T *__restrict__ zero_rows,
+                                                   const int pu,  // prefix of the thread within its chunk
+                                                   T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW>::kStage],
+                                                   T (&slot)[ForwardShape<T, D, N, P, GW>::kSlots]
+                                                            [ForwardShape<T, D, N, P, GW>::kSlotSize]) {
     using G = Geometry<D, N, P>;
     constexpr int KS = N - P;
-    constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
-    constexpr int kSlotSize = GW > 1 ? (int)G::kSigSize : 4;
-    __shared__ __align__(16) T sdx_all[GW][kTile * KS * D];
-    __shared__ __align__(16) T slot[kSlots][kSlotSize];
     const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
-    const int pu = (int)threadIdx.x - part * G::kBlock;
     T *sdx = sdx_all[part];
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
@@ -569,11 +647,11 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
             int tt = 0;
             for (; tt + 1 < nt; tt += 2) {
                 read_increments<T, D, P, KS>(sdx, tt + 1, u, dxs1, dxp1);
-                StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
+                StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
                 read_increments<T, D, P, KS>(sdx, tt + 2 < nt ? tt + 2 : tt + 1, u, dxs0, dxp0);
-                StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs1, dxp1);
+                StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs1, dxp1);
             }
-            if (tt < nt) StepTargets<T, D, P, N, false>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
+            if (tt < nt) StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
         }
     }
     if constexpr (GW > 1) {
@@ -591,6 +669,30 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
         if (part == 0 && active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
     } else {
         if (active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
+    }
+}
+
+// BOUNDED: `bounds` holds the letter bounds of the wanted top-level words (see LetterBounds).  Every wave runs
+// the copy of the sweep compiled for its bound; the copies differ in nothing but the sub-trie nodes they leave
+// out, so all waves of the block still meet at the same barriers.
+template <typename T, int D, int N, int P, int GW, bool BOUNDED = false>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
+    dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
+                         T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr) {
+    using FS = ForwardShape<T, D, N, P, GW>;
+    static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
+    __shared__ __align__(16) T sdx_all[GW][FS::kStage];
+    __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
+    const int tid = (int)threadIdx.x % Geometry<D, N, P>::kBlock;
+    if constexpr (BOUNDED) {
+        const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
+        const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
+        dispatch_value<0, D>(lo, [&](auto loc) {
+            dense_forward_body<T, D, N, P, GW, decltype(loc)::value>(path, out, shape, chunks, zero_rows, pu, sdx_all,
+                                                                     slot);
+        });
+    } else {
+        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, tid, sdx_all, slot);
     }
 }
 
@@ -836,22 +938,35 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     }
 }
 
-template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
-    dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
-                          const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
-                          SigShape shape, int chunks, T *__restrict__ grad_path = nullptr) {
+// LDS layout of the reverse sweep.  Per-increment sums leave a wave as four row sums; the tile flush adds the
+// parts of all waves in a fixed order.  The tile is shortened until the parts fit 48 KB of LDS.
+template <typename T, int D, int N, int P>
+struct BackwardShape {
     using G = Geometry<D, N, P>;
+    static constexpr int KS = N - P;
+    static constexpr int kParts = 4;
+    static constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
+    static constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32 : 16;
+    static constexpr int kStage = kBwdTile * KS * D;
+    static constexpr int kSums = G::kWaves * kParts;
+    static constexpr int kSumRow = kBwdTile * D;
+};
+
+// BOUND: the upstream gradient is zero on every top-level word that has a letter below BOUND after the
+// prefix's first letter, and the sweep leaves those words out; the LDS arrays belong to the calling kernel.
+template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, int BOUND>
+__device__ __forceinline__ void dense_backward_body(
+    const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig, const T *__restrict__ edgeA,
+    const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
+    const int pu,  // prefix of the thread
+    T (&sdx)[BackwardShape<T, D, N, P>::kStage],
+    T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow]) {
+    using G = Geometry<D, N, P>;
+    using BS = BackwardShape<T, D, N, P>;
     constexpr int KS = N - P;
-    // per-increment sums leave a wave as four row sums; the tile flush adds the parts of all waves in a
-    // fixed order.  The tile is shortened until the parts fit 48 KB of LDS.
-    constexpr int kParts = 4;
+    constexpr int kParts = BS::kParts;
+    constexpr int kBwdTile = BS::kBwdTile;
     constexpr bool kToPath = CHUNKED && !ACCUMULATE;  // writes the path gradient itself (see the tile flush)
-    constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
-    constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32 : 16;
-    __shared__ __align__(16) T sdx[kBwdTile * KS * D];
-    __shared__ T sg[G::kWaves * kParts][kBwdTile * D];
-    const int pu = threadIdx.x;
     const int lane = pu & (kWave - 1);
     const int wave = pu / kWave;
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
@@ -915,7 +1030,8 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
                 for (int k = 0; k < D; ++k) gdxk[q][k] = T(0);
 #pragma unroll
             for (int j = 0; j < P; ++j) gpre[j] = T(0);
-            AdjTargets<T, D, N, P, 1>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
+            AdjTargets<T, D, N, P, 1, BOUND>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxp, gdxk,
+                                                                                gpre);
             // letter k collects the sub-trie sums (with the 1/(q+1) of their increments) and the chain
             // positions whose letter is k
             T tot[D];
@@ -1010,6 +1126,32 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     }
 }
 
+// BOUNDED: the upstream gradient is zero on every top-level word outside the letter bounds in `bounds` (see
+// LetterBounds).  Every wave runs the copy of the sweep compiled for its bound; all copies meet at the same
+// barriers.
+template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, bool BOUNDED = false>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+    dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
+                          const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
+                          SigShape shape, int chunks, T *__restrict__ grad_path = nullptr,
+                          const int *__restrict__ bounds = nullptr) {
+    using BS = BackwardShape<T, D, N, P>;
+    static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
+    __shared__ __align__(16) T sdx[BS::kStage];
+    __shared__ T sg[BS::kSums][BS::kSumRow];
+    if constexpr (BOUNDED) {
+        const int pu = LetterBounds<D, P>::prefix_of_thread((int)threadIdx.x);
+        const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
+        dispatch_value<0, D>(lo, [&](auto loc) {
+            dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value>(
+                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, sdx, sg);
+        });
+    } else {
+        dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0>(path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape,
+                                                                chunks, grad_path, (int)threadIdx.x, sdx, sg);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side: table of compiled shapes and launch sequences
 // ---------------------------------------------------------------------------------------------
@@ -1024,12 +1166,28 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 struct VariantInfo {
     int d, depth, block;
     int64_t sig_size, low_size;
+    bool bounds_ok;  // the sweeps can leave out top-level words by letter bounds
 };
 
 template <int D, int N, int P>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
-    return VariantInfo{D, N, G::kBlock, G::kSigSize, G::kLowSize};
+    return VariantInfo{D, N, G::kBlock, G::kSigSize, G::kLowSize, LetterBounds<D, P>::kUsable && D <= 16};
+}
+
+constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
+
+// Computes the letter bounds of the top-level word list into the head of *workspace and moves *workspace
+// past them; returns nullptr (and launches nothing) when the call does not use bounds.
+const int *stage_letter_bounds(const DenseChoice &dc, const int64_t *top_codes, int64_t top_count, int d, int depth,
+                               void **workspace, hipStream_t stream) {
+    if (!dc.bounded) return nullptr;
+    int *bounds = (int *)*workspace;
+    *workspace = (unsigned char *)*workspace + kBoundsBytes;
+    const bool narrow = (double)depth * std::log2((double)d) < 32.0;
+    hipLaunchKernelGGL(letter_bounds_kernel, dim3(1), dim3(1024), 0, stream, top_codes, top_count, d, depth, narrow,
+                       bounds);
+    return bounds;
 }
 
 #define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P>(),
@@ -1073,12 +1231,22 @@ constexpr bool group_fits() {
 }
 
 template <typename T, int D, int N, int P, int PC>
-hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, void *workspace, hipStream_t stream) {
+hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, void *workspace,
+                       hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
     const int64_t rows = shape.B * shape.W;
+    if (bounds && !kBoundsOk) return hipErrorInvalidValue;
     if (chunks <= 1) {
+        if constexpr (kBoundsOk) {
+            if (bounds) {
+                hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)rows), dim3(G::kBlock),
+                                   0, stream, path, sig, shape, 1, (T *)nullptr, bounds);
+                return hipGetLastError();
+            }
+        }
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
                            path, sig, shape, 1);
         return hipGetLastError();
@@ -1087,6 +1255,14 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     // a row that fits one block goes straight to the output, without the combine launch
     T *chunk_sig = (T *)workspace;
     int groups = chunks;
+    if constexpr (kBoundsOk) {
+        if (bounds) {
+            // bounded sweeps exist one chunk to a block only
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)(rows * chunks)),
+                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds);
+            groups = -1;
+        }
+    }
     if constexpr (group_fits<T, D, N, P, 4>()) {
         if (groups == chunks && chunks % 4 == 0) {
             groups = chunks / 4;
@@ -1106,6 +1282,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            stream, path, chunk_sig, shape, chunks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || groups == 1) return e;
+    if (groups < 0) groups = chunks;
     if constexpr (kStaged)
         hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, true>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
                            (const T *)chunk_sig, sig, groups);
@@ -1117,13 +1294,16 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
 
 template <typename T, int D, int N, int P, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
-                        const SigShape &shape, int chunks, void *workspace, hipStream_t stream) {
+                        const SigShape &shape, int chunks, const int *bounds, void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PS>;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
     const int64_t rows = shape.B * shape.W;
     const bool accumulate = shape.windows != nullptr;
     *wrote_path = false;
     hipError_t e;
+    // bounded sweeps exist for time-chunked calls only (every call that embeds a projection is chunked)
+    if (bounds && (!kBoundsOk || chunks <= 1)) return hipErrorInvalidValue;
     if (accumulate) {
         e = launch_fill_zero<T>(grad_inc, shape.B * (shape.L - 1) * shape.d, stream);
         if (e != hipSuccess) return e;
@@ -1178,16 +1358,31 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         profile_mark(true, stream);
-        if (accumulate) {
-            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units), dim3(G::kBlock),
-                               0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH, grad_inc, shape,
-                               chunks, (T *)nullptr);
-        } else {
-            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
-                               dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
-                               grad_inc, shape, chunks, grad_path);
-            *wrote_path = true;
+        bool launched = false;
+        if constexpr (kBoundsOk) {
+            if (bounds) {
+                if (accumulate)
+                    hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true, true>), dim3((unsigned)units),
+                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA,
+                                       (const T *)dumpH, grad_inc, shape, chunks, (T *)nullptr, bounds);
+                else
+                    hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true, true>), dim3((unsigned)units),
+                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA,
+                                       (const T *)dumpH, grad_inc, shape, chunks, grad_path, bounds);
+                launched = true;
+            }
         }
+        if (!launched) {
+            if (accumulate)
+                hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units),
+                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
+                                   grad_inc, shape, chunks, (T *)nullptr);
+            else
+                hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
+                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
+                                   grad_inc, shape, chunks, grad_path);
+        }
+        if (!accumulate) *wrote_path = true;
         profile_mark(false, stream);
         return hipGetLastError();
     }
@@ -1229,6 +1424,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             if ((double)rows * (double)v.sig_size * (double)elem > 4e9) return dc;
             dc.embed = true;
             dc.dense_bytes = pad256((size_t)rows * v.sig_size * elem);
+            dc.bounded = v.bounds_ok && level_sizes[depth] > 0 && level_sizes[depth] < top_dense &&
+                         !getenv("PATHSIG_NO_LETTER_BOUNDS");
         }
         int chunks = pick_chunks(rows, v.block, L);
         if (const char *env = getenv("PATHSIG_CHUNKS")) {
@@ -1240,8 +1437,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         dc.variant = i;
         dc.fwd_chunks = chunks;
         dc.bwd_chunks = (dc.embed && chunks < 2) ? 2 : chunks;
-        dc.forward_workspace = dc.dense_bytes;
-        dc.backward_workspace = dc.dense_bytes;
+        dc.forward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
+        dc.backward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
         if (dc.fwd_chunks > 1) dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem);
         if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
         return dc;
@@ -1250,15 +1447,18 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
 }
 
 #define PSIG_CASE_FWD(I, D, N, P, PC, PS) \
-    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, workspace, stream);
+    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, workspace, stream);
 #define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
     case I:                                                                                                        \
         return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc.bwd_chunks, \
-                                            workspace, stream);
+                                            bounds, workspace, stream);
 
 template <typename T>
-hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc, void *workspace,
-                                hipStream_t stream) {
+hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
+                                const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream) {
+    if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
+    const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
+                                            kVariants[dc.variant].depth, &workspace, stream);
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_FWD)
         default: return hipErrorNotSupported;
@@ -1267,19 +1467,22 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
 
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
-                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc, void *workspace,
-                                 hipStream_t stream) {
+                                 bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
+                                 const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream) {
+    if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
+    const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
+                                            kVariants[dc.variant].depth, &workspace, stream);
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_BWD)
         default: return hipErrorNotSupported;
     }
 }
 
-#define PSIG_INSTANTIATE(T)                                                                                    \
-    template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const DenseChoice &, void *,  \
-                                                hipStream_t);                                                  \
+#define PSIG_INSTANTIATE(T)                                                                                      \
+    template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const DenseChoice &,            \
+                                                const int64_t *, int64_t, void *, hipStream_t);                  \
     template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, T *, bool *, const SigShape &, \
-                                                 const DenseChoice &, void *, hipStream_t);
+                                                 const DenseChoice &, const int64_t *, int64_t, void *, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE

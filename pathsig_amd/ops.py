@@ -60,7 +60,13 @@ def _host_i64(values: Sequence[int]):
     return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
 
 
+# handle of the current stream without building a torch.cuda.Stream object (about 2 us less per call)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device: torch.device) -> ctypes.c_void_p:
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

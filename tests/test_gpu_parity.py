@@ -5,6 +5,8 @@ fp64 1e-12, fp32 1e-5, as the build target states.  Index and layout checks are 
 """
 from __future__ import annotations
 
+import random
+
 import pytest
 import torch
 
@@ -625,3 +627,42 @@ def test_logsignature_lyndon_through_dense_kernels(ps, dtype):
     xr = path.clone().requires_grad_(True)
     (want_grad,) = torch.autograd.grad(TO.logsignature(xr, depth).index_select(-1, cols), xr, G)
     assert rel_err(grad, want_grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("kind", ["irregular", "lyndon"])
+def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dtype, kind):
+    """d = 8, depth 5: the sweeps leave out the top-level words whose later letters fall below the
+    smallest one used after the same first letter.  The word list has a different bound per first letter,
+    one first letter without words, and unordered, repeated words; the run without bounds must agree."""
+    import itertools
+    d, depth, B, L = 8, 5, 2, 45
+    if kind == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    else:
+        least = {0: 0, 1: 3, 2: 8, 3: 1, 5: 6, 6: 7, 7: 2}   # first letter -> smallest later letter (4: no words)
+        rng = random.Random(12)
+        top = []
+        for first, lo in least.items():
+            if lo >= d:
+                continue
+            tails = list(itertools.product(range(lo, d), repeat=depth - 1))
+            keep = tails if first == 0 else rng.sample(tails, min(len(tails), 300))
+            top += [(first,) + t for t in keep]
+            top.append((first,) + (lo,) * (depth - 1))       # the bound is attained
+        rng.shuffle(top)
+        top += top[:5]
+        proj = ps.projections.words(top, depth=depth, path_dim=d, full_levels=(1, 2, 3, 4))
+    sizes, codes = _plan(proj)
+    assert sizes[depth] * 8 >= d ** depth and sizes[depth] < d ** depth
+    path = brownian_path(B, L, d, seed=91) * 1.5
+    for windows in (None, [(0, 45), (7, 30), (20, 22)]):
+        want = TO.compute_signature(path, depth, sizes, codes, windows)
+        G = randn(tuple(want.shape), seed=92)
+        got, grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[dtype]
+        assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes, windows)) < TOL[dtype]
+        monkeypatch.setenv("PATHSIG_NO_LETTER_BOUNDS", "1")
+        plain, plain_grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
+        monkeypatch.delenv("PATHSIG_NO_LETTER_BOUNDS")
+        assert rel_err(got, plain) < TOL[dtype] and rel_err(grad, plain_grad) < TOL[dtype]
