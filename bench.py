@@ -205,6 +205,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the extra leg that captures one step in a HIP graph and times replays of it "
+                         "(reported beside the eager figure as graph_replay; `value` is always the eager one)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also copy one 256 MiB buffer once (untimed), as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -241,14 +244,17 @@ def main():
         torch.autograd.grad(out, xg, G)
 
     # whole-step throughput: W warm-up steps, then exactly K steps between synchronisations
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    def time_steps(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    elapsed = time_steps(step)
     ms_per_step = 1e3 * elapsed / args.steps
 
     fwd_mean, fwd_med = time_events(fwd_only, args.steps, 3)
@@ -268,6 +274,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}, {args.dtype}",
                    "step": "forward + backward" if cfg["backward"] else "forward",
+                   "launch": "eager",
                    "out_shape": list(wl["out_shape"]), "horner_nodes_per_increment": wl["nodes"]},
         "fwd_paths_per_s": B / (fwd_med * 1e-3),
         "fwd_ms": fwd_med,
@@ -320,6 +327,26 @@ def main():
             result["roofline"] = dict(result["roofline_backward_call"])
     else:
         result["roofline"] = dict(result["roofline_forward"], kernel="signature forward call")
+    if not args.no_graph:
+        # the same step captured once in a HIP graph and replayed: what a caller gets who takes the Python and
+        # launch overhead out of the loop (the library neither allocates nor synchronises, so it captures)
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            replay_ms = 1e3 * time_steps(graph.replay) / args.steps
+            result["graph_replay"] = {"ms_per_step": replay_ms, "value": B / (replay_ms * 1e-3), "unit": "paths/s",
+                                      "step_frac_of_peak": step_flops / (replay_ms * 1e-3) / 1e12 / peak}
+            del graph
+        except Exception as exc:  # a capture failure must not cost the eager figures
+            result["graph_replay"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl, dtype)
     print(json.dumps(result))
