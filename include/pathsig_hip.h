@@ -74,6 +74,27 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same pair with a hand-over from the forward to the backward of one call (no counterpart in the
+ * reference, whose backward receives the path and the signature only and recomputes what it needs).
+ * On long paths the register-tiled kernels cut every row into time chunks; the forward can write the
+ * signature of each chunk below the top level into `chunks`, and a backward that is given the same buffer
+ * skips the launch that would recompute them.  pathsig_sig_chunks_bytes() returns the size of that buffer
+ * for a call, or 0 when the call has nothing to hand over (then use the plain entry points).  All other
+ * arguments are as above; `chunks == NULL` makes both functions identical to the plain ones.
+ */
+size_t pathsig_sig_chunks_bytes(int dtype, int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                                int64_t W);
+int pathsig_sig_forward_keep(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                             const int64_t *level_sizes, const int64_t *encoded_words, int64_t n_encoded,
+                             const int32_t *windows, int64_t W, void *chunks, size_t chunks_bytes, void *workspace,
+                             size_t workspace_bytes, void *stream);
+int pathsig_sig_backward_kept(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                              int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                              const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                              const void *chunks, size_t chunks_bytes, void *workspace, size_t workspace_bytes,
+                              void *stream);
+
+/*
  * Signature -> log-signature on the hybrid layout (levels 1..depth-1 dense, level `depth` with
  * `top_size` columns whose codes are `top_words`, a DEVICE int64 array, or NULL when the top level
  * is dense).  Replaces sig_to_logsig (src/pathsig/forward/sig_launch.cu:230-339, op

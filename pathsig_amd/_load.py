@@ -14,7 +14,7 @@ import threading
 import torch
 
 _LIB_NAME = "libpathsig_hip.so"
-_ABI_VERSION = 1
+_ABI_VERSION = 2
 _lock = threading.Lock()
 _lib: ctypes.CDLL | None = None
 
@@ -45,6 +45,14 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pathsig_sig_backward.restype = _INT
     lib.pathsig_sig_backward.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _I64, _INT, _PTR, _PTR, _I64,
                                          _PTR, _I64, _PTR, _SIZE, _PTR]
+    lib.pathsig_sig_chunks_bytes.restype = _SIZE
+    lib.pathsig_sig_chunks_bytes.argtypes = [_INT, _I64, _I64, _I64, _INT, _PTR, _I64]
+    lib.pathsig_sig_forward_keep.restype = _INT
+    lib.pathsig_sig_forward_keep.argtypes = [_PTR, _PTR, _INT, _I64, _I64, _I64, _INT, _PTR, _PTR, _I64, _PTR, _I64,
+                                             _PTR, _SIZE, _PTR, _SIZE, _PTR]
+    lib.pathsig_sig_backward_kept.restype = _INT
+    lib.pathsig_sig_backward_kept.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _I64, _INT, _PTR, _PTR, _I64,
+                                              _PTR, _I64, _PTR, _SIZE, _PTR, _SIZE, _PTR]
     lib.pathsig_logsig_forward.restype = _INT
     lib.pathsig_logsig_forward.argtypes = [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _I64, _PTR, _PTR]
     lib.pathsig_logsig_backward_workspace.restype = _SIZE

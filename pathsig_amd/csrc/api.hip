@@ -125,8 +125,8 @@ int launch_failed(hipError_t e, const char *what) {
 
 template <typename T>
 int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
-                  const int64_t *codes, int64_t n_encoded, const int32_t *windows, int64_t W, void *workspace,
-                  size_t workspace_bytes, hipStream_t stream) {
+                  const int64_t *codes, int64_t n_encoded, const int32_t *windows, int64_t W, void *keep,
+                  size_t keep_bytes, void *workspace, size_t workspace_bytes, hipStream_t stream) {
     LevelPlan plan;
     bool all_dense;
     int rc = build_plan(d, depth, level_sizes, n_encoded, codes != nullptr, &plan, &all_dense);
@@ -136,6 +136,10 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
     rc = check_grid(plan, B * shape.W);
     if (rc != PATHSIG_OK) return rc;
     const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
+    if (keep && (!dc.usable || dc.keep_bytes == 0 || keep_bytes < dc.keep_bytes)) {
+        set_error("chunk buffer: this call keeps %zu bytes, got %zu", dc.usable ? dc.keep_bytes : (size_t)0, keep_bytes);
+        return PATHSIG_ERR_ARGUMENT;
+    }
     if (dc.usable) {
         if (workspace_bytes < dc.forward_workspace || (dc.forward_workspace && !workspace)) {
             set_error("workspace too small: need %zu bytes, got %zu", dc.forward_workspace, workspace_bytes);
@@ -145,8 +149,8 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
         T *dense = dc.embed ? (T *)workspace : (T *)sig;
         void *rest = (unsigned char *)workspace + dc.dense_bytes;
         const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
-        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, top_codes, plan.size[depth], rest,
-                                               stream);
+        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, top_codes, plan.size[depth], (T *)keep,
+                                               rest, stream);
         if (e != hipSuccess) return launch_failed(e, "dense forward launch");
         if (dc.embed) {
             e = launch_gather_columns<T>(dense, (T *)sig, plan, d, codes, B * shape.W, stream);
@@ -162,7 +166,8 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
 template <typename T>
 int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void *grad_path, int64_t B, int64_t L,
                    int64_t d, int depth, const int64_t *level_sizes, const int64_t *codes, int64_t n_encoded,
-                   const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+                   const int32_t *windows, int64_t W, const void *kept, size_t kept_bytes, void *workspace,
+                   size_t workspace_bytes, hipStream_t stream) {
     LevelPlan plan;
     bool all_dense;
     int rc = build_plan(d, depth, level_sizes, n_encoded, codes != nullptr, &plan, &all_dense);
@@ -172,6 +177,10 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     rc = check_grid(plan, B * shape.W);
     if (rc != PATHSIG_OK) return rc;
     const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
+    if (kept && (!dc.usable || dc.keep_bytes == 0 || kept_bytes < dc.keep_bytes)) {
+        set_error("chunk buffer: this call keeps %zu bytes, got %zu", dc.usable ? dc.keep_bytes : (size_t)0, kept_bytes);
+        return PATHSIG_ERR_ARGUMENT;
+    }
     const size_t inc_bytes = align_up((size_t)(B * (L - 1) * d) * sizeof(T));
     const size_t need = inc_bytes + (dc.usable ? dc.backward_workspace : 0);
     if (!workspace || workspace_bytes < need) {
@@ -197,7 +206,7 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
         const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
         e = launch_dense_backward<T>((const T *)path, dc.embed ? (const T *)nullptr : (const T *)sig, gdense, ginc,
                                      (T *)grad_path, &wrote_path, shape, dc, top_codes, plan.size[depth],
-                                     extra + dc.dense_bytes, stream);
+                                     (const T *)kept, extra + dc.dense_bytes, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
         if (wrote_path) return PATHSIG_OK;
     } else {
@@ -256,7 +265,7 @@ using namespace psig;
 
 extern "C" {
 
-int pathsig_abi_version(void) { return 1; }
+int pathsig_abi_version(void) { return 2; }
 
 const char *pathsig_last_error(void) { return g_error; }
 
@@ -278,9 +287,28 @@ size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d,
     return dc.usable ? dc.forward_workspace : 0;
 }
 
+size_t pathsig_sig_chunks_bytes(int dtype, int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                                int64_t W) {
+    if (check_common(dtype, B, L, d, depth) != PATHSIG_OK) return 0;
+    LevelPlan plan;
+    bool all_dense;
+    if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
+    const DenseChoice dc =
+        dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
+    return dc.usable ? dc.keep_bytes : 0;
+}
+
 int pathsig_sig_forward(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,
                         const int64_t *level_sizes, const int64_t *encoded_words, int64_t n_encoded,
                         const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes, void *stream) {
+    return pathsig_sig_forward_keep(path, sig, dtype, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows,
+                                    W, nullptr, 0, workspace, workspace_bytes, stream);
+}
+
+int pathsig_sig_forward_keep(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,
+                             const int64_t *level_sizes, const int64_t *encoded_words, int64_t n_encoded,
+                             const int32_t *windows, int64_t W, void *chunks, size_t chunks_bytes, void *workspace,
+                             size_t workspace_bytes, void *stream) {
     int rc = check_common(dtype, B, L, d, depth);
     if (rc != PATHSIG_OK) return rc;
     if (B > 0 && (!path || !sig)) {
@@ -293,9 +321,9 @@ int pathsig_sig_forward(const void *path, void *sig, int dtype, int64_t B, int64
     }
     if (dtype == PATHSIG_F32)
         return sig_forward_t<float>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W,
-                                    workspace, workspace_bytes, (hipStream_t)stream);
-    return sig_forward_t<double>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W,
-                                 workspace, workspace_bytes, (hipStream_t)stream);
+                                    chunks, chunks_bytes, workspace, workspace_bytes, (hipStream_t)stream);
+    return sig_forward_t<double>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W, chunks,
+                                 chunks_bytes, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
@@ -313,6 +341,15 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
                          int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
                          const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
                          void *workspace, size_t workspace_bytes, void *stream) {
+    return pathsig_sig_backward_kept(path, sig, grad_sig, grad_path, dtype, B, L, d, depth, level_sizes, encoded_words,
+                                     n_encoded, windows, W, nullptr, 0, workspace, workspace_bytes, stream);
+}
+
+int pathsig_sig_backward_kept(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                              int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                              const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                              const void *chunks, size_t chunks_bytes, void *workspace, size_t workspace_bytes,
+                              void *stream) {
     int rc = check_common(dtype, B, L, d, depth);
     if (rc != PATHSIG_OK) return rc;
     if (B > 0 && (!path || !grad_path)) {
@@ -325,9 +362,11 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
     }
     if (dtype == PATHSIG_F32)
         return sig_backward_t<float>(path, sig, grad_sig, grad_path, B, L, d, depth, level_sizes, encoded_words,
-                                     n_encoded, windows, W, workspace, workspace_bytes, (hipStream_t)stream);
+                                     n_encoded, windows, W, chunks, chunks_bytes, workspace, workspace_bytes,
+                                     (hipStream_t)stream);
     return sig_backward_t<double>(path, sig, grad_sig, grad_path, B, L, d, depth, level_sizes, encoded_words,
-                                  n_encoded, windows, W, workspace, workspace_bytes, (hipStream_t)stream);
+                                  n_encoded, windows, W, chunks, chunks_bytes, workspace, workspace_bytes,
+                                  (hipStream_t)stream);
 }
 
 int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, int64_t rows, int64_t d, int depth,

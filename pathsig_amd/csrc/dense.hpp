@@ -15,6 +15,7 @@ struct DenseChoice {
     size_t dense_bytes;         // embed: bytes of one dense [rows, S] buffer
     size_t forward_workspace;   // bytes of scratch the forward needs (including the dense buffer)
     size_t backward_workspace;  // bytes of scratch the backward needs beyond the increment accumulator
+    size_t keep_bytes;          // bytes of chunk signatures the forward can keep for the backward (0: none)
 };
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,
@@ -22,15 +23,19 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
 
 // `sig` / `grad_sig` are dense-layout rows; `workspace` is the part of the scratch after any dense buffer.
 // top_codes / top_count: the word list of the top level (device memory), read only when dc.bounded.
+// keep (optional, dc.keep_bytes bytes): receives the signatures of the time chunks below the top level; passing
+// the same buffer as `kept` to the backward of the same call saves it the launch that recomputes them.
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
-                                const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream);
+                                const int64_t *top_codes, int64_t top_count, T *keep, void *workspace,
+                                hipStream_t stream);
 // The backward fills grad_inc ([B, L-1, d] increment gradients), or, for time-chunked calls without windows,
 // writes grad_path ([B, L, d]) itself and reports that in *wrote_path.
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                  bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
-                                 const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream);
+                                 const int64_t *top_codes, int64_t top_count, const T *kept, void *workspace,
+                                 hipStream_t stream);
 
 // measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
 // the begin and the end of that kernel on its stream; a no-op while the hook is off)

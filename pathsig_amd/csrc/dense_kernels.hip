@@ -576,10 +576,7 @@ constexpr size_t forward_lds_bytes() {
     return (size_t)GW * kTile * (N - P) * D * sizeof(T) + (size_t)(GW / 2) * G::kSigSize * sizeof(T);
 }
 
-// zero_rows (optional, GW = 1): the block also clears the points of its chunk in a [B, L, D] buffer (the last
-// chunk of a row clears the final point too); the backward uses this to prepare the path gradient.
-// BOUND: top-level words with a letter below BOUND after the prefix's first letter are left out (they stay zero
-// in the output); the LDS arrays belong to the calling kernel.
+// LDS layout of the forward sweep: staged increments per chunk, and slots for the in-block products
 template <typename T, int D, int N, int P, int GW>
 struct ForwardShape {
     using G = Geometry<D, N, P>;
@@ -589,9 +586,15 @@ struct ForwardShape {
     static constexpr int kStage = kTile * KS * D;  // staged increments of one chunk
 };
 
+// zero_rows (optional, GW = 1): the block also clears the points of its chunk in a [B, L, D] buffer (the last
+// chunk of a row clears the final point too); the backward uses this to prepare the path gradient.
+// chunk_low (optional): [rows, chunks, levels below N] receives every chunk's own signature below the top level.
+// BOUND: top-level words with a letter below BOUND after the prefix's first letter are left out (they stay zero
+// in the output); the LDS arrays belong to the calling kernel.
 template <typename T, int D, int N, int P, int GW, int BOUND>
 __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T *__restrict__ out,
                                                    const SigShape &shape, int chunks, T *__restrict__ zero_rows,
+                                                   T *__restrict__ chunk_low,
                                                    const int pu,  // prefix of the thread within its chunk
                                                    T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW>::kStage],
                                                    T (&slot)[ForwardShape<T, D, N, P, GW>::kSlots]
@@ -654,6 +657,11 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             if (tt < nt) StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
         }
     }
+    if constexpr (N - 1 >= P) {
+        // the chunk's own signature below the top level, kept for the backward of the same call
+        if (chunk_low != nullptr && active)
+            store_state<T, D, P, N - 1, G::kFwdSub>(chunk_low + (row * chunks + c) * G::kLowSize, pu, a, sub);
+    }
     if constexpr (GW > 1) {
         const SubWords<D, P> sw(u);
 #pragma unroll
@@ -678,7 +686,8 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
 template <typename T, int D, int N, int P, int GW, bool BOUNDED = false>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
-                         T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr) {
+                         T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr,
+                         T *__restrict__ chunk_low = nullptr) {
     using FS = ForwardShape<T, D, N, P, GW>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
@@ -688,11 +697,11 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
         const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
-            dense_forward_body<T, D, N, P, GW, decltype(loc)::value>(path, out, shape, chunks, zero_rows, pu, sdx_all,
-                                                                     slot);
+            dense_forward_body<T, D, N, P, GW, decltype(loc)::value>(path, out, shape, chunks, zero_rows, chunk_low, pu,
+                                                                     sdx_all, slot);
         });
     } else {
-        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, tid, sdx_all, slot);
+        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, chunk_low, tid, sdx_all, slot);
     }
 }
 
@@ -1231,8 +1240,8 @@ constexpr bool group_fits() {
 }
 
 template <typename T, int D, int N, int P, int PC>
-hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, void *workspace,
-                       hipStream_t stream) {
+hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, T *keep,
+                       void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
@@ -1259,7 +1268,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
         if (bounds) {
             // bounded sweeps exist one chunk to a block only
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)(rows * chunks)),
-                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds);
+                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds, keep);
             groups = -1;
         }
     }
@@ -1267,19 +1276,21 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
         if (groups == chunks && chunks % 4 == 0) {
             groups = chunks / 4;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 4>), dim3((unsigned)(rows * groups)),
-                               dim3(G::kBlock * 4), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks);
+                               dim3(G::kBlock * 4), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks,
+                               (T *)nullptr, (const int *)nullptr, keep);
         }
     }
     if constexpr (group_fits<T, D, N, P, 2>()) {
         if (groups == chunks && chunks % 2 == 0) {
             groups = chunks / 2;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 2>), dim3((unsigned)(rows * groups)),
-                               dim3(G::kBlock * 2), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks);
+                               dim3(G::kBlock * 2), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks,
+                               (T *)nullptr, (const int *)nullptr, keep);
         }
     }
     if (groups == chunks)
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0,
-                           stream, path, chunk_sig, shape, chunks);
+                           stream, path, chunk_sig, shape, chunks, (T *)nullptr, (const int *)nullptr, keep);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || groups == 1) return e;
     if (groups < 0) groups = chunks;
@@ -1294,7 +1305,8 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
 
 template <typename T, int D, int N, int P, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
-                        const SigShape &shape, int chunks, const int *bounds, void *workspace, hipStream_t stream) {
+                        const SigShape &shape, int chunks, const int *bounds, const T *kept, void *workspace,
+                        hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PS>;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
@@ -1332,13 +1344,22 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         T *dumpA = (T *)ws;
         ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpH = (T *)ws;
-        // chunk signatures below the top level: the depth N-1 forward kernel on the same units
-        // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
-        hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P, 1>), dim3((unsigned)units),
-                           dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks,
-                           accumulate ? (T *)nullptr : grad_path);
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        if (kept) {
+            // the forward of this call kept its chunk signatures: only the path gradient is left to clear
+            chunk_low = const_cast<T *>(kept);
+            if (!accumulate) {
+                e = launch_fill_zero<T>(grad_path, shape.B * shape.L * shape.d, stream);
+                if (e != hipSuccess) return e;
+            }
+        } else {
+            // chunk signatures below the top level: the depth N-1 forward kernel on the same units
+            // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P, 1>), dim3((unsigned)units),
+                               dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks,
+                               accumulate ? (T *)nullptr : grad_path);
+            e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
         // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
         const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
         const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
@@ -1441,22 +1462,27 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         dc.backward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
         if (dc.fwd_chunks > 1) dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem);
         if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
+        // the forward can hand its chunk signatures to the backward when both cut the rows the same way
+        if (dc.bwd_chunks > 1 && dc.fwd_chunks == dc.bwd_chunks)
+            dc.keep_bytes = (size_t)rows * dc.bwd_chunks * v.low_size * elem;
         return dc;
     }
     return dc;
 }
 
 #define PSIG_CASE_FWD(I, D, N, P, PC, PS) \
-    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, workspace, stream);
+    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace, stream);
 #define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
     case I:                                                                                                        \
         return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc.bwd_chunks, \
-                                            bounds, workspace, stream);
+                                            bounds, kept, workspace, stream);
 
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
-                                const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream) {
+                                const int64_t *top_codes, int64_t top_count, T *keep, void *workspace,
+                                hipStream_t stream) {
     if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
+    if (keep && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
     switch (dc.variant) {
@@ -1468,8 +1494,10 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                  bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
-                                 const int64_t *top_codes, int64_t top_count, void *workspace, hipStream_t stream) {
+                                 const int64_t *top_codes, int64_t top_count, const T *kept, void *workspace,
+                                 hipStream_t stream) {
     if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
+    if (kept && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
     switch (dc.variant) {
@@ -1480,9 +1508,10 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
 
 #define PSIG_INSTANTIATE(T)                                                                                      \
     template hipError_t launch_dense_forward<T>(const T *, T *, const SigShape &, const DenseChoice &,            \
-                                                const int64_t *, int64_t, void *, hipStream_t);                  \
+                                                const int64_t *, int64_t, T *, void *, hipStream_t);             \
     template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, T *, bool *, const SigShape &, \
-                                                 const DenseChoice &, const int64_t *, int64_t, void *, hipStream_t);
+                                                 const DenseChoice &, const int64_t *, int64_t, const T *, void *,  \
+                                                 hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE

@@ -8,6 +8,7 @@ and hands raw pointers plus the current HIP stream to the C ABI declared in incl
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Sequence
 
 import torch
@@ -31,6 +32,16 @@ _library.define(
 _library.define(
     "sig_to_logsig(Tensor signature_in, int depth, int d, bool alternative_projection, Tensor encoded_words, "
     "int[] level_sizes) -> (Tensor, Tensor)", tags=_PT2)
+# The same signature pair with a hand-over from the forward to the backward (not in the reference): the forward
+# also returns the signatures of its time chunks below the top level (an empty tensor when the call is not
+# time-chunked), and the backward that receives them skips the launch that would recompute them.
+_library.define(
+    "compute_signature_keep(Tensor path_in, int depth, bool alternative_projection, Tensor encoded_words, "
+    "int[] level_sizes, bool use_windows, Tensor windows) -> (Tensor, Tensor)", tags=_PT2)
+_library.define(
+    "signature_backward_kept(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, Tensor chunks, int depth, "
+    "bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, Tensor windows) -> Tensor",
+    tags=_PT2)
 _library.define(
     "logsig_backward(Tensor signature_in, Tensor P_in, Tensor grad_logsig_in, int depth, "
     "bool alternative_projection, Tensor encoded_words, int[] level_sizes) -> Tensor", tags=_PT2)
@@ -95,8 +106,15 @@ def _windows_arg(windows: Tensor) -> Tensor:
 # ------------------------------------------------------------------------------------------------
 # device implementations (dispatch key CUDA == HIP on ROCm builds)
 # ------------------------------------------------------------------------------------------------
-@torch.library.impl(_library, "compute_signature", "CUDA")
-def _compute_signature_hip(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows):
+def _chunks_numel(path: Tensor, depth: int, alternative_projection: bool, level_sizes, W: int) -> int:
+    """Elements of the chunk buffer a forward on `path` can hand to its backward (0: nothing to hand over)."""
+    B, L, d = (int(n) for n in path.shape)
+    sizes_host = _host_i64(level_sizes) if alternative_projection else None
+    nbytes = _load.lib().pathsig_sig_chunks_bytes(_dtype_code(path), B, L, d, int(depth), sizes_host, int(W))
+    return int(nbytes) // path.element_size()
+
+
+def _sig_forward(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows, keep):
     _require(path_in.is_cuda, "path must be CUDA")
     _require(path_in.dim() == 3, "path must be [B,T,d]")
     dt = _dtype_code(path_in)
@@ -119,20 +137,37 @@ def _compute_signature_hip(path_in, depth, alternative_projection, encoded_words
     W = int(win.size(0)) if win is not None else 0
     out = torch.empty((B, W, sig_size) if use_windows else (B, sig_size), dtype=path.dtype, device=path.device)
     lib = _load.lib()
+    chunks = None
     with torch.cuda.device(path.device):
+        if keep:
+            n_keep = lib.pathsig_sig_chunks_bytes(dt, B, L, d, depth, sizes_host, W) // path.element_size()
+            chunks = torch.empty(n_keep, dtype=path.dtype, device=path.device)
         ws_bytes = lib.pathsig_sig_forward_workspace(dt, B, L, d, depth, sizes_host, W)
         ws = _scratch(ws_bytes, path.device)
-        rc = lib.pathsig_sig_forward(
+        rc = lib.pathsig_sig_forward_keep(
             _ptr(path), _ptr(out), dt, B, L, d, depth, sizes_host, _ptr(words), 0 if words is None else words.numel(),
-            _ptr(win) if use_windows else None, W, _ptr(ws), ws_bytes, _stream(path.device))
+            _ptr(win) if use_windows else None, W, _ptr(chunks), 0 if chunks is None else chunks.numel() * chunks.element_size(),
+            _ptr(ws), ws_bytes, _stream(path.device))
     if rc != 0:
         _fail(rc)
-    return out
+    return out, chunks
 
 
-@torch.library.impl(_library, "signature_backward", "CUDA")
-def _signature_backward_hip(path_in, signature_in, grad_signature_in, depth, alternative_projection, encoded_words,
-                            level_sizes, use_windows, windows):
+@torch.library.impl(_library, "compute_signature", "CUDA")
+def _compute_signature_hip(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows):
+    return _sig_forward(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows,
+                        keep=False)[0]
+
+
+@torch.library.impl(_library, "compute_signature_keep", "CUDA")
+def _compute_signature_keep_hip(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows,
+                                windows):
+    return _sig_forward(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows,
+                        keep=True)
+
+
+def _sig_backward(path_in, signature_in, grad_signature_in, chunks, depth, alternative_projection, encoded_words,
+                  level_sizes, use_windows, windows):
     _require(path_in.is_cuda, "path must be CUDA")
     _require(path_in.dim() == 3, "path must be [B,T,d]")
     dt = _dtype_code(path_in)
@@ -171,16 +206,35 @@ def _signature_backward_hip(path_in, signature_in, grad_signature_in, depth, alt
         _require(sig.dim() == 2, "signature must be [B,S] when no windows are used")
     out = torch.empty_like(path)
     lib = _load.lib()
+    if chunks is not None and chunks.numel() > 0:
+        _require(chunks.is_cuda and chunks.dtype == path.dtype, "chunks must be a CUDA tensor of the path's dtype")
+        chunks = chunks.contiguous()
+    else:
+        chunks = None
     with torch.cuda.device(path.device):
         ws_bytes = lib.pathsig_sig_backward_workspace(dt, B, L, d, depth, sizes_host, W)
         ws = _scratch(ws_bytes, path.device)
-        rc = lib.pathsig_sig_backward(
+        rc = lib.pathsig_sig_backward_kept(
             _ptr(path), _ptr(sig), _ptr(grad), _ptr(out), dt, B, L, d, depth, sizes_host, _ptr(words),
-            0 if words is None else words.numel(), _ptr(win) if use_windows else None, W, _ptr(ws), ws_bytes,
-            _stream(path.device))
+            0 if words is None else words.numel(), _ptr(win) if use_windows else None, W, _ptr(chunks),
+            0 if chunks is None else chunks.numel() * chunks.element_size(), _ptr(ws), ws_bytes, _stream(path.device))
     if rc != 0:
         _fail(rc)
     return out
+
+
+@torch.library.impl(_library, "signature_backward", "CUDA")
+def _signature_backward_hip(path_in, signature_in, grad_signature_in, depth, alternative_projection, encoded_words,
+                            level_sizes, use_windows, windows):
+    return _sig_backward(path_in, signature_in, grad_signature_in, None, depth, alternative_projection, encoded_words,
+                         level_sizes, use_windows, windows)
+
+
+@torch.library.impl(_library, "signature_backward_kept", "CUDA")
+def _signature_backward_kept_hip(path_in, signature_in, grad_signature_in, chunks, depth, alternative_projection,
+                                 encoded_words, level_sizes, use_windows, windows):
+    return _sig_backward(path_in, signature_in, grad_signature_in, chunks, depth, alternative_projection, encoded_words,
+                         level_sizes, use_windows, windows)
 
 
 def _hybrid_top(signature: Tensor, depth: int, d: int, alternative_projection: bool, level_sizes):
@@ -269,7 +323,13 @@ def _logsig_backward_hip(signature_in, P_in, grad_logsig_in, depth, alternative_
 # ------------------------------------------------------------------------------------------------
 def compute_signature(path: Tensor, depth: int, alternative_projection: bool, encoded_words: Tensor,
                       level_sizes: list[int], use_windows: bool, windows: Tensor) -> Tensor:
-    """(Windowed / projected) signature of a batch of paths."""
+    """(Windowed / projected) signature of a batch of paths.
+
+    When a gradient will be asked for, the forward also keeps what its backward would otherwise recompute
+    (the signatures of the time chunks of long paths); the values returned are the same either way."""
+    if torch.is_grad_enabled() and path.requires_grad and not os.environ.get("PATHSIG_NO_KEEP"):
+        return torch.ops.pathsig.compute_signature_keep.default(
+            path, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows)[0]
     return torch.ops.pathsig.compute_signature.default(
         path, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows)
 
@@ -349,6 +409,24 @@ def _compute_signature_fake(path, depth, alternative_projection, encoded_words, 
     return torch.empty(shape, device=path.device, dtype=path.dtype)
 
 
+@torch.library.register_fake("pathsig::compute_signature_keep", lib=_library)
+def _compute_signature_keep_fake(path, depth, alternative_projection, encoded_words, level_sizes, use_windows,
+                                 windows):
+    out = _compute_signature_fake(path, depth, alternative_projection, encoded_words, level_sizes, use_windows,
+                                  windows)
+    n_keep = _chunks_numel(path, depth, alternative_projection, level_sizes, windows.size(0) if use_windows else 0)
+    return out, torch.empty((n_keep,), device=path.device, dtype=path.dtype)
+
+
+@torch.library.register_fake("pathsig::signature_backward_kept", lib=_library)
+def _signature_backward_kept_fake(path, signature, grad_signature, chunks, depth, alternative_projection,
+                                  encoded_words, level_sizes, use_windows, windows):
+    torch._check(_on_device(chunks))
+    torch._check(chunks.dim() == 1)
+    return _signature_backward_fake(path, signature, grad_signature, depth, alternative_projection, encoded_words,
+                                    level_sizes, use_windows, windows)
+
+
 @torch.library.register_fake("pathsig::sig_to_logsig", lib=_library)
 def _sig_to_logsig_fake(signature, depth, d, alternative_projection, encoded_words, level_sizes):
     torch._check(_on_device(signature), lambda: "signature must be a CUDA tensor")
@@ -421,6 +499,27 @@ def _signature_vjp(ctx, grad_out):
 
 torch.library.register_autograd("pathsig::compute_signature", _signature_vjp, setup_context=_save_for_signature,
                                 lib=_library)
+
+
+def _save_for_signature_keep(ctx, inputs, output):
+    path, depth, alt, encoded_words, level_sizes, use_windows, windows = inputs
+    signature, chunks = output
+    ctx.save_for_backward(path, signature, chunks, windows, encoded_words)
+    ctx.depth, ctx.alt, ctx.level_sizes, ctx.use_windows = int(depth), bool(alt), level_sizes, bool(use_windows)
+
+
+def _signature_keep_vjp(ctx, grad_out, grad_chunks):
+    path, signature, chunks, windows, encoded_words = ctx.saved_tensors
+    grad_path = None
+    if ctx.needs_input_grad[0]:
+        grad_path = torch.ops.pathsig.signature_backward_kept.default(
+            path, signature, grad_out, chunks, ctx.depth, ctx.alt, encoded_words, ctx.level_sizes, ctx.use_windows,
+            windows)
+    return grad_path, None, None, None, None, None, None
+
+
+torch.library.register_autograd("pathsig::compute_signature_keep", _signature_keep_vjp,
+                                setup_context=_save_for_signature_keep, lib=_library)
 
 
 def _save_for_logsig(ctx, inputs, output):

@@ -27,10 +27,11 @@ def test_header_functions_are_exported(lib):
     names = declared_functions()
     assert {"pathsig_sig_forward", "pathsig_sig_backward", "pathsig_logsig_forward", "pathsig_logsig_backward",
             "pathsig_sig_forward_workspace", "pathsig_sig_backward_workspace", "pathsig_logsig_backward_workspace",
+            "pathsig_sig_chunks_bytes", "pathsig_sig_forward_keep", "pathsig_sig_backward_kept",
             "pathsig_last_error", "pathsig_abi_version"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
-    assert lib.pathsig_abi_version() == 1
+    assert lib.pathsig_abi_version() == 2
 
 
 def _fwd(lib, dtype=0, B=2, L=5, d=3, depth=3, path=1, sig=1, sizes=None):

@@ -666,3 +666,64 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dt
         plain, plain_grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
         monkeypatch.delenv("PATHSIG_NO_LETTER_BOUNDS")
         assert rel_err(got, plain) < TOL[dtype] and rel_err(grad, plain_grad) < TOL[dtype]
+
+
+# ------------------------------------------------------------------------------------------------
+# hand-over of the time-chunk signatures from the forward to the backward of one call
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("case", ["dense", "windows", "lyndon", "not_chunked", "per_word"])
+def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, case):
+    """`compute_signature_keep` / `signature_backward_kept` (what the modules use when a gradient is wanted)
+    against the reference's pair `compute_signature` / `signature_backward`: same signature, same dL/dpath,
+    whether or not the call is time-chunked (the chunk buffer is empty when it is not)."""
+    import ctypes
+    from pathsig_amd import _load
+    depth, kw, chunked = 4, {}, True
+    if case == "dense":
+        d, B, L = 4, 5, 300
+        monkeypatch.setenv("PATHSIG_CHUNKS", "5")
+    elif case == "windows":
+        d, B, L = 4, 3, 200
+        kw["windows"] = [(0, 200), (10, 150), (40, 42), (7, 7)]
+        monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+    elif case == "lyndon":
+        d, depth, B, L = 8, 5, 2, 90
+        kw["projection"] = ps.projections.lyndon(depth=depth, path_dim=d, full_levels=(1, 2, 3, 4))
+        monkeypatch.setenv("PATHSIG_CHUNKS", "3")
+    elif case == "not_chunked":
+        d, B, L, chunked = 4, 3000, 20, False
+    else:
+        d, B, L, chunked = 5, 3, 40, False          # no register-tiled shape for d = 5: per-word kernels
+    path = brownian_path(B, L, d, seed=401) * 1.5
+    x = path.to(dtype).to(DEV)
+    wins = kw.get("windows")
+    mod = ps.Signature(depth=depth, projection=kw.get("projection"),
+                       windows=None if wins is None else torch.tensor(wins, dtype=torch.int64, device=DEV))
+    args = (mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes, mod.use_windows, mod._windows)
+    sig = torch.ops.pathsig.compute_signature(x, *args)
+    G = randn(tuple(sig.shape), seed=402).to(dtype).to(DEV)
+    grad = torch.ops.pathsig.signature_backward(x, sig, G, *args)
+    sig_k, chunks = torch.ops.pathsig.compute_signature_keep(x, *args)
+    assert (chunks.numel() > 0) == chunked
+    sizes = None if not mod.alternative_projection else (ctypes.c_int64 * len(mod._level_sizes))(*mod._level_sizes)
+    assert chunks.numel() * chunks.element_size() == _load.lib().pathsig_sig_chunks_bytes(
+        0 if dtype == torch.float32 else 1, B, L, d, depth, sizes, 0 if wins is None else len(wins))
+    grad_k = torch.ops.pathsig.signature_backward_kept(x, sig_k, G, chunks, *args)
+    assert torch.equal(sig_k, sig)
+    assert rel_err(grad_k, grad) < TOL[dtype] * 0.1
+    # the module takes the keeping pair when a gradient is wanted
+    xg = x.clone().requires_grad_(True)
+    out = mod(xg)
+    assert out.grad_fn is not None and "Keep" in type(out.grad_fn).__name__.replace("keep", "Keep")
+    (grad_m,) = torch.autograd.grad(out, xg, G)
+    assert torch.equal(out.detach(), sig) and rel_err(grad_m, grad) < TOL[dtype] * 0.1
+    # a chunk buffer of the wrong size is refused
+    if chunked:
+        with pytest.raises(RuntimeError, match="chunk buffer"):
+            torch.ops.pathsig.signature_backward_kept(x, sig, G, chunks[:-1], *args)
+    checks = ("test_schema", "test_faketensor", "test_autograd_registration")
+    if case in ("dense", "per_word") and dtype == torch.float64:
+        torch.library.opcheck(torch.ops.pathsig.compute_signature_keep.default, (xg, *args), test_utils=checks)
+        torch.library.opcheck(torch.ops.pathsig.signature_backward_kept.default, (x, sig, G, chunks, *args),
+                              test_utils=checks)
