@@ -8,6 +8,7 @@ There is no fallback: if the library is missing, importing the package fails.
 from __future__ import annotations
 
 import ctypes
+import os
 import pathlib
 import threading
 
@@ -91,3 +92,24 @@ def ensure_loaded() -> ctypes.CDLL:
 
 def lib() -> ctypes.CDLL:
     return ensure_loaded()
+
+
+_TORCH_LIB_NAME = "libpathsig_torch.so"
+_torch_ops_loaded: bool | None = None
+
+
+def load_torch_ops() -> bool:
+    """Loads the C++ registration of the operators (schemas, device implementations, autograd) if it is built.
+
+    Returns False when it is absent or `PATHSIG_PYTHON_OPS=1` asks for the registration from Python; both
+    run the same kernels of libpathsig_hip.so, the C++ one without the interpreter's overhead per call."""
+    global _torch_ops_loaded
+    if _torch_ops_loaded is None:
+        ensure_loaded()
+        path = pathlib.Path(__file__).resolve().parent / _TORCH_LIB_NAME
+        if os.environ.get("PATHSIG_PYTHON_OPS") or not path.is_file():
+            _torch_ops_loaded = False
+        else:
+            torch.ops.load_library(str(path))
+            _torch_ops_loaded = True
+    return _torch_ops_loaded

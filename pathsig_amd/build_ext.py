@@ -1,7 +1,9 @@
-"""Compiles pathsig_amd/csrc/*.hip for gfx950 into pathsig_amd/libpathsig_hip.so with hipcc.
+"""Compiles pathsig_amd/csrc/*.hip for gfx950 into pathsig_amd/libpathsig_hip.so with hipcc, and the torch
+operator registration csrc/torch_ops.cpp into pathsig_amd/libpathsig_torch.so with g++.
 
-Run `python -m pathsig_amd.build_ext` (or `__graft_entry__.build()`).  No torch headers are needed:
-the library is a plain C-ABI shared object declared in include/pathsig_hip.h.
+Run `python pathsig_amd/build_ext.py` (or `__graft_entry__.build()`).  The first library needs no torch headers:
+it is a plain C-ABI shared object declared in include/pathsig_hip.h.  The second one links against it and against
+the torch libraries of the running interpreter.
 """
 from __future__ import annotations
 
@@ -14,6 +16,7 @@ PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB = PKG / "libpathsig_hip.so"
+TORCH_LIB = PKG / "libpathsig_torch.so"
 
 SOURCES = ["api.hip", "words_kernels.hip", "batch_kernels.hip", "logsig_kernels.hip", "dense_kernels.hip"]
 
@@ -57,5 +60,29 @@ def build(verbose: bool = False, jobs: int = 4) -> pathlib.Path:
     return LIB
 
 
+def build_torch_ops(verbose: bool = False) -> pathlib.Path:
+    """C++ registration of the operators with the torch dispatcher (host code only; needs libpathsig_hip.so)."""
+    import torch
+    from torch.utils import cpp_extension
+
+    if torch.version.hip is None:
+        raise RuntimeError("the operator library needs a ROCm build of PyTorch")
+    includes = [f"-I{p}" for p in cpp_extension.include_paths()] + ["-I/opt/rocm/include", f"-I{INCLUDE}"]
+    lib_dirs = cpp_extension.library_paths()
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", *includes,
+           str(CSRC / "torch_ops.cpp"), "-o", str(TORCH_LIB),
+           *[f"-L{d}" for d in lib_dirs], "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+           f"-L{PKG}", "-lpathsig_hip", "-Wl,-rpath,$ORIGIN", *[f"-Wl,-rpath,{d}" for d in lib_dirs]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("g++ failed on torch_ops.cpp")
+    return TORCH_LIB
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_torch_ops(verbose=True))

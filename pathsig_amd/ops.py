@@ -20,31 +20,42 @@ __all__ = ["compute_signature", "sig_to_logsig", "signature_backward", "logsig_b
 
 _F32, _F64 = 0, 1
 
-_library = torch.library.Library("pathsig", "DEF")
+# The C++ registration (csrc/torch_ops.cpp: schemas, device implementations and autograd nodes) is used when
+# it is built; otherwise the same is registered from Python below.  Shape inference for fake tensors is
+# registered from Python in both cases.
+_NATIVE_OPS = _load.load_torch_ops()
+_library = torch.library.Library("pathsig", "FRAGMENT" if _NATIVE_OPS else "DEF")
 _PT2 = (torch.Tag.pt2_compliant_tag,)
-_library.define(
-    "compute_signature(Tensor path_in, int depth, bool alternative_projection, Tensor encoded_words, "
-    "int[] level_sizes, bool use_windows, Tensor windows) -> Tensor", tags=_PT2)
-_library.define(
-    "signature_backward(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, int depth, "
-    "bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, Tensor windows) -> Tensor",
-    tags=_PT2)
-_library.define(
-    "sig_to_logsig(Tensor signature_in, int depth, int d, bool alternative_projection, Tensor encoded_words, "
-    "int[] level_sizes) -> (Tensor, Tensor)", tags=_PT2)
-# The same signature pair with a hand-over from the forward to the backward (not in the reference): the forward
-# also returns the signatures of its time chunks below the top level (an empty tensor when the call is not
-# time-chunked), and the backward that receives them skips the launch that would recompute them.
-_library.define(
-    "compute_signature_keep(Tensor path_in, int depth, bool alternative_projection, Tensor encoded_words, "
-    "int[] level_sizes, bool use_windows, Tensor windows) -> (Tensor, Tensor)", tags=_PT2)
-_library.define(
-    "signature_backward_kept(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, Tensor chunks, int depth, "
-    "bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, Tensor windows) -> Tensor",
-    tags=_PT2)
-_library.define(
-    "logsig_backward(Tensor signature_in, Tensor P_in, Tensor grad_logsig_in, int depth, "
-    "bool alternative_projection, Tensor encoded_words, int[] level_sizes) -> Tensor", tags=_PT2)
+
+
+def _define_schemas() -> None:
+    _library.define(
+        "compute_signature(Tensor path_in, int depth, bool alternative_projection, Tensor encoded_words, "
+        "int[] level_sizes, bool use_windows, Tensor windows) -> Tensor", tags=_PT2)
+    _library.define(
+        "signature_backward(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, int depth, "
+        "bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, Tensor windows) -> Tensor",
+        tags=_PT2)
+    _library.define(
+        "sig_to_logsig(Tensor signature_in, int depth, int d, bool alternative_projection, Tensor encoded_words, "
+        "int[] level_sizes) -> (Tensor, Tensor)", tags=_PT2)
+    # The same signature pair with a hand-over from the forward to the backward (not in the reference): the forward
+    # also returns the signatures of its time chunks below the top level (an empty tensor when the call is not
+    # time-chunked), and the backward that receives them skips the launch that would recompute them.
+    _library.define(
+        "compute_signature_keep(Tensor path_in, int depth, bool alternative_projection, Tensor encoded_words, "
+        "int[] level_sizes, bool use_windows, Tensor windows) -> (Tensor, Tensor)", tags=_PT2)
+    _library.define(
+        "signature_backward_kept(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, Tensor chunks, int depth, "
+        "bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, Tensor windows) -> Tensor",
+        tags=_PT2)
+    _library.define(
+        "logsig_backward(Tensor signature_in, Tensor P_in, Tensor grad_logsig_in, int depth, "
+        "bool alternative_projection, Tensor encoded_words, int[] level_sizes) -> Tensor", tags=_PT2)
+
+
+if not _NATIVE_OPS:
+    _define_schemas()
 
 
 # ------------------------------------------------------------------------------------------------
@@ -153,13 +164,11 @@ def _sig_forward(path_in, depth, alternative_projection, encoded_words, level_si
     return out, chunks
 
 
-@torch.library.impl(_library, "compute_signature", "CUDA")
 def _compute_signature_hip(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows):
     return _sig_forward(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows,
                         keep=False)[0]
 
 
-@torch.library.impl(_library, "compute_signature_keep", "CUDA")
 def _compute_signature_keep_hip(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows,
                                 windows):
     return _sig_forward(path_in, depth, alternative_projection, encoded_words, level_sizes, use_windows, windows,
@@ -223,14 +232,12 @@ def _sig_backward(path_in, signature_in, grad_signature_in, chunks, depth, alter
     return out
 
 
-@torch.library.impl(_library, "signature_backward", "CUDA")
 def _signature_backward_hip(path_in, signature_in, grad_signature_in, depth, alternative_projection, encoded_words,
                             level_sizes, use_windows, windows):
     return _sig_backward(path_in, signature_in, grad_signature_in, None, depth, alternative_projection, encoded_words,
                          level_sizes, use_windows, windows)
 
 
-@torch.library.impl(_library, "signature_backward_kept", "CUDA")
 def _signature_backward_kept_hip(path_in, signature_in, grad_signature_in, chunks, depth, alternative_projection,
                                  encoded_words, level_sizes, use_windows, windows):
     return _sig_backward(path_in, signature_in, grad_signature_in, chunks, depth, alternative_projection, encoded_words,
@@ -249,7 +256,6 @@ def _hybrid_top(signature: Tensor, depth: int, d: int, alternative_projection: b
     return top
 
 
-@torch.library.impl(_library, "sig_to_logsig", "CUDA")
 def _sig_to_logsig_hip(signature_in, depth, d, alternative_projection, encoded_words, level_sizes):
     _require(signature_in.is_cuda, "signature must be CUDA")
     dt = _dtype_code(signature_in)
@@ -278,7 +284,6 @@ def _sig_to_logsig_hip(signature_in, depth, d, alternative_projection, encoded_w
     return logsig, P
 
 
-@torch.library.impl(_library, "logsig_backward", "CUDA")
 def _logsig_backward_hip(signature_in, P_in, grad_logsig_in, depth, alternative_projection, encoded_words, level_sizes):
     _require(signature_in.is_cuda, "sig must be CUDA")
     _require(P_in.is_cuda, "P must be CUDA")
@@ -497,8 +502,6 @@ def _signature_vjp(ctx, grad_out):
     return grad_path, None, None, None, None, None, None
 
 
-torch.library.register_autograd("pathsig::compute_signature", _signature_vjp, setup_context=_save_for_signature,
-                                lib=_library)
 
 
 def _save_for_signature_keep(ctx, inputs, output):
@@ -518,8 +521,6 @@ def _signature_keep_vjp(ctx, grad_out, grad_chunks):
     return grad_path, None, None, None, None, None, None
 
 
-torch.library.register_autograd("pathsig::compute_signature_keep", _signature_keep_vjp,
-                                setup_context=_save_for_signature_keep, lib=_library)
 
 
 def _save_for_logsig(ctx, inputs, output):
@@ -538,4 +539,17 @@ def _logsig_vjp(ctx, grad_logsig, grad_cache):
     return grad_sig, None, None, None, None, None
 
 
-torch.library.register_autograd("pathsig::sig_to_logsig", _logsig_vjp, setup_context=_save_for_logsig, lib=_library)
+if not _NATIVE_OPS:
+    for _name, _impl in (("compute_signature", _compute_signature_hip),
+                         ("compute_signature_keep", _compute_signature_keep_hip),
+                         ("signature_backward", _signature_backward_hip),
+                         ("signature_backward_kept", _signature_backward_kept_hip),
+                         ("sig_to_logsig", _sig_to_logsig_hip),
+                         ("logsig_backward", _logsig_backward_hip)):
+        _library.impl(_name, _impl, "CUDA")
+    torch.library.register_autograd("pathsig::compute_signature", _signature_vjp, setup_context=_save_for_signature,
+                                    lib=_library)
+    torch.library.register_autograd("pathsig::compute_signature_keep", _signature_keep_vjp,
+                                    setup_context=_save_for_signature_keep, lib=_library)
+    torch.library.register_autograd("pathsig::sig_to_logsig", _logsig_vjp, setup_context=_save_for_logsig,
+                                    lib=_library)
