@@ -858,7 +858,8 @@ __device__ __forceinline__ void copy_row_out(const T *src_lds, T *__restrict__ d
 // for the whole scan); otherwise they stream through a double buffer, one chunk ahead.
 template <typename T, int D, int N, int P, bool RESIDENT>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
-    dense_scan_kernel(const T *__restrict__ chunk_low, T *__restrict__ edgeA, T *__restrict__ edgeZ, int chunks) {
+    dense_scan_kernel(const T *__restrict__ chunk_low, T *__restrict__ edgeA, T *__restrict__ edgeZ, int chunks,
+                      T *__restrict__ zero_rows = nullptr, int64_t row_elems = 0) {
     using G = Geometry<D, N, P>;
     using Stager = RowStager<T, (int)G::kLowSize, G::kBlock>;
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
@@ -876,6 +877,15 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     prefix_letters<D, P>(active ? pu : 0, u);
     const SubWords<D, P> sw(u);
     const int64_t row = blockIdx.x;
+    if (zero_rows) {
+        // the two blocks of a row clear one half each of the row's row_elems values in a second buffer (the path
+        // gradient, which the reverse sweep then accumulates into)
+        const int64_t half = (row_elems + 1) / 2;
+        const int64_t first = (int64_t)blockIdx.y * half;
+        const int64_t last = first + half < row_elems ? first + half : row_elems;
+        T *z = zero_rows + row * row_elems;
+        for (int64_t i = first + threadIdx.x; i < last; i += kThreads) z[i] = T(0);
+    }
     const T *rows = chunk_low + row * chunks * kLow;
     const int last = chunks - 1;
     if constexpr (RESIDENT) {
@@ -1345,12 +1355,8 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         ws += pad256((size_t)units * G::kLowSize * sizeof(T));
         T *dumpH = (T *)ws;
         if (kept) {
-            // the forward of this call kept its chunk signatures: only the path gradient is left to clear
+            // the forward of this call kept its chunk signatures; the scan launch below clears the path gradient
             chunk_low = const_cast<T *>(kept);
-            if (!accumulate) {
-                e = launch_fill_zero<T>(grad_path, shape.B * shape.L * shape.d, stream);
-                if (e != hipSuccess) return e;
-            }
         } else {
             // chunk signatures below the top level: the depth N-1 forward kernel on the same units
             // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
@@ -1360,6 +1366,9 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             e = hipGetLastError();
             if (e != hipSuccess) return e;
         }
+        // without windows rows are paths: with kept chunk signatures the scan clears the path gradient
+        T *clear = (kept && !accumulate) ? grad_path : (T *)nullptr;
+        const int64_t clear_elems = shape.L * shape.d;
         // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
         const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
         const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
@@ -1371,10 +1380,11 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), resident_bytes, stream,
-                               (const T *)chunk_low, dumpA, dumpH, chunks);
+                               (const T *)chunk_low, dumpA, dumpH, chunks, clear, clear_elems);
         } else {
             hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS, false>), dim3((unsigned)rows, 2),
-                               dim3(GC::kBlock + kCopyThreads), 0, stream, (const T *)chunk_low, dumpA, dumpH, chunks);
+                               dim3(GC::kBlock + kCopyThreads), 0, stream, (const T *)chunk_low, dumpA, dumpH, chunks,
+                               clear, clear_elems);
         }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
