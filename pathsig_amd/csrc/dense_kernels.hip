@@ -1178,9 +1178,12 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 // of length P, the per-row combine kernel on prefixes of length PC and the per-row scan kernel (which
 // works on levels below N) on prefixes of length PS.  The backward also runs the forward kernel of
 // depth N-1 (same P) to get chunk signatures below the top level.
+// A (D, N) listed twice: the entry with the shorter prefix comes first and is taken when the call has enough
+// rows to fill the GPU with it; otherwise the longer prefix (more lanes per row, a few more chain FMAs per
+// lane) is taken.
 #define PSIG_VARIANTS(X) \
     X(0, 4, 6, 3, 5, 4) X(1, 8, 4, 2, 3, 2) X(2, 6, 5, 3, 3, 3) X(3, 4, 4, 2, 3, 2) X(4, 3, 5, 3, 4, 3) \
-    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3)
+    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3) X(7, 8, 4, 3, 3, 2)
 
 struct VariantInfo {
     int d, depth, block;
@@ -1360,8 +1363,10 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         } else {
             // chunk signatures below the top level: the depth N-1 forward kernel on the same units
             // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
-            hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, P, 1>), dim3((unsigned)units),
-                               dim3(Geometry<D, N - 1, P>::kBlock), 0, stream, path, chunk_low, shape, chunks,
+            // (the forward kernel needs a prefix shorter than its depth; the layout it writes does not depend on it)
+            constexpr int PK = P <= N - 2 ? P : N - 2;
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, PK, 1>), dim3((unsigned)units),
+                               dim3(Geometry<D, N - 1, PK>::kBlock), 0, stream, path, chunk_low, shape, chunks,
                                accumulate ? (T *)nullptr : grad_path);
             e = hipGetLastError();
             if (e != hipSuccess) return e;
@@ -1446,6 +1451,14 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         const VariantInfo &v = kVariants[i];
         if (v.d != d || v.depth != depth) continue;
         const int64_t rows = B * W;
+        {
+            // a later entry for the same (d, depth) has more lanes per row: take it when this one cannot
+            // put about a wave on every SIMD even with the most time chunks the path allows
+            bool later = false;
+            for (int j = i + 1; j < kNumVariants; ++j) later = later || (kVariants[j].d == d && kVariants[j].depth == depth);
+            const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
+            if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
+        }
         if (!all_dense) {
             // A word projection is worth computing densely when its top level keeps a fair share of the
             // words (the top level dominates the cost) and the dense rows fit comfortably in memory.

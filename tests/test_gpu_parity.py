@@ -727,3 +727,20 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, cas
         torch.library.opcheck(torch.ops.pathsig.compute_signature_keep.default, (xg, *args), test_utils=checks)
         torch.library.opcheck(torch.ops.pathsig.signature_backward_kept.default, (x, sig, G, chunks, *args),
                               test_utils=checks)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("chunks", [None, "4"])
+def test_shape_with_two_prefix_lengths(ps, monkeypatch, dtype, chunks):
+    """(d, depth) = (8, 4) is compiled with lanes on prefixes of length 2 and of length 3; small batches take the
+    longer prefix (the other tests of this shape), a batch that fills the GPU takes the shorter one."""
+    if chunks:
+        monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
+    d, depth, B, L = 8, 4, 200, 100
+    path = brownian_path(B, L, d, seed=501)
+    for windows in (None, [(0, 100), (10, 90), (50, 52)]):
+        want = TO.compute_signature(path, depth, windows=windows)
+        G = randn(tuple(want.shape), seed=502)
+        got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[dtype]
+        assert rel_err(grad, TO.signature_vjp(path, G, depth, windows=windows)) < TOL[dtype]
