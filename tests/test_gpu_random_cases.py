@@ -1,0 +1,93 @@
+"""Seeded random cases against the level-tensor checker: shapes with and without a register-tiled kernel,
+both dtypes, windows (degenerate ones included), every projection builder, forced time-chunk counts, through the
+modules (forward that keeps its chunk signatures) and through the reference's stateless pair of ops."""
+from __future__ import annotations
+
+import itertools
+import random
+
+import pytest
+import torch
+
+from oracle import tensor_oracle as TO
+from tests.helpers import brownian_path, randn, random_word_set, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (8, 5)]
+OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 6), (16, 3), (9, 3), (4, 5), (6, 3)]
+
+
+def _random_case(rng, ps):
+    d, depth = rng.choice(TILED) if rng.random() < 0.6 else rng.choice(OTHER)
+    small = d ** depth < 5000
+    B = rng.choice([1, 2, 3, 5, 17, 40]) if small else rng.choice([1, 2, 3])
+    L = rng.choice([2, 3, 7, 33, 65, 130, 200]) if small else rng.choice([2, 5, 40, 70])
+    dtype = rng.choice([torch.float32, torch.float64])
+    kind = rng.choice(["dense", "dense", "lyndon", "words", "top_words", "aniso"])
+    windows = None
+    if rng.random() < 0.4:
+        windows = []
+        for _ in range(rng.randint(1, 6)):
+            start = rng.randint(0, L - 1)
+            windows.append((start, rng.randint(start, L)))
+    chunks = rng.choice([None, None, "2", "3", "7"])
+    proj = None
+    if kind == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    elif kind == "words":
+        count = rng.randint(1, min(60, sum(d ** k for k in range(1, depth + 1))))
+        proj = ps.projections.words(random_word_set(d, 1, depth, count, seed=rng.randint(0, 999)), depth=depth,
+                                    path_dim=d)
+    elif kind == "top_words":
+        n_top = max(1, int(d ** depth * rng.choice([0.05, 0.2, 0.6])))
+        top = rng.sample(list(itertools.product(range(d), repeat=depth)), min(n_top, d ** depth - 1))
+        if rng.random() < 0.5:
+            top = top + top[:3]
+        proj = ps.projections.words(top, depth=depth, path_dim=d, full_levels=tuple(range(1, depth)))
+    elif kind == "aniso":
+        weights = [rng.choice([1.0, 1.5, 2.0, 3.0]) for _ in range(d)]
+        try:
+            proj = ps.projections.anisotropic(weights, weight_threshold=rng.choice([3.0, 4.5, 6.0]), depth=depth,
+                                              path_dim=d)
+        except ValueError:
+            proj = None
+    scale = rng.choice([0.5, 1.0, 2.0])
+    seeds = (rng.randint(0, 10 ** 6), rng.randint(0, 10 ** 6))
+    return d, depth, B, L, dtype, proj, windows, chunks, scale, seeds
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_signature_cases(monkeypatch, seed):
+    import pathsig_amd as ps
+    rng = random.Random(seed)
+    for case in range(40):
+        d, depth, B, L, dtype, proj, windows, chunks, scale, seeds = _random_case(rng, ps)
+        if d ** depth > 40000:
+            continue
+        if chunks:
+            monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
+        else:
+            monkeypatch.delenv("PATHSIG_CHUNKS", raising=False)
+        sizes, codes = (None, None) if proj is None else (proj.level_sizes, proj._codes)
+        path = brownian_path(B, L, d, seed=seeds[0]) * scale
+        want = TO.compute_signature(path, depth, sizes, codes, windows)
+        G = randn(tuple(want.shape), seed=seeds[1])
+        try:
+            want_grad = TO.signature_vjp(path, G, depth, sizes, codes, windows)
+        except RuntimeError:  # every window degenerate: the checker's output does not depend on the path
+            want_grad = torch.zeros_like(path)
+        tol = 1e-5 if dtype == torch.float32 else 1e-12
+        what = f"seed {seed} case {case}: d={d} depth={depth} B={B} L={L} {dtype} windows={windows} chunks={chunks}"
+        x = path.to(dtype).to(DEV).requires_grad_(True)
+        win = None if windows is None else torch.tensor(windows, dtype=torch.int64, device=DEV)
+        mod = ps.Signature(depth=depth, projection=proj, windows=win)
+        out = mod(x)
+        (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+        assert rel_err(out, want) < tol and rel_err(grad, want_grad) < tol, what
+        args = (mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes, mod.use_windows,
+                mod._windows)
+        with torch.no_grad():
+            sig = torch.ops.pathsig.compute_signature(x, *args)
+            grad = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)
+        assert rel_err(sig, want) < tol and rel_err(grad, want_grad) < tol, what
