@@ -334,13 +334,16 @@ __global__ void logsig_q_kernel(const T *__restrict__ P, T *__restrict__ Q_all, 
     }
 }
 
-// Levels below the top, one block per row.  `a` ([lower columns][depth], workspace) holds a_m, `R` ([lower
-// columns], workspace) the top-level sums of logsig_gather_top_kernel, which has also stored the top-level
-// part of the gradient in grad_sig.
+// Levels below the top, one block per row.  `a` ([lower columns][depth]) holds a_m: in LDS when the launch
+// provides room for it (a_in_lds; the kernel is a chain of short dependent passes over `a`, so their latency is
+// what it costs), else in the workspace.  `R` ([lower columns], workspace) are the top-level sums of
+// logsig_gather_top_kernel, which has also stored the top-level part of the gradient in grad_sig.
 template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ sig, const T *__restrict__ P,
                                                                   const T *__restrict__ grad_logsig, T *grad_sig,
-                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp) {
+                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp,
+                                                                  int a_in_lds) {
+    extern __shared__ __align__(16) unsigned char gather_smem[];
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
     const int64_t row = blockIdx.x;
@@ -348,7 +351,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     const T *Pr = P + row * hp.total * N;
     const T *gl = grad_logsig + row * hp.total;
     T *gs = grad_sig + row * hp.total;
-    T *a = a_all + row * hp.lower * N;
+    T *a = a_in_lds ? reinterpret_cast<T *>(gather_smem) : a_all + row * hp.lower * N;
     const T *R = R_all + row * hp.lower;
     int64_t width[kMaxDepth + 1];  // d^k
     width[0] = 1;
@@ -525,8 +528,16 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
                            stream, sig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, P, grad_logsig,
-                           grad_sig, gradP, (const T *)R, hp);
+        // the adjoint of the cache goes to LDS when a block's share of it fits beside the static arrays
+        const size_t a_bytes = (size_t)hp.lower * (size_t)depth * sizeof(T);
+        const bool a_in_lds = a_bytes <= 144 * 1024;
+        if (a_in_lds && a_bytes > 32 * 1024) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_kernel<T>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)a_bytes);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), a_in_lds ? a_bytes : 0, stream,
+                           sig, P, grad_logsig, grad_sig, gradP, (const T *)R, hp, a_in_lds ? 1 : 0);
         return hipGetLastError();
     }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
