@@ -969,6 +969,13 @@ struct BackwardShape {
     static constexpr int kStage = kBwdTile * KS * D;
     static constexpr int kSums = G::kWaves * kParts;
     static constexpr int kSumRow = kBwdTile * D;
+    // fp64: the chain's P terms reach their letters through LDS (a row of D cells per lane, letter-major so that
+    // a wave's accesses never share a bank).  A lane's prefix never changes, so it only ever touches the same
+    // P cells and the others stay zero: P LDS adds, D loads and P clearing stores replace 3 * P * D selects and
+    // adds of a kernel that is bound by vector instruction issue.  fp32 multiplies by one-hot constants instead
+    // where those fit the register file.
+    static constexpr bool kChainCells = sizeof(T) == 8 && D <= 8 && D * G::kBlock * (int)sizeof(T) <= 32 * 1024;
+    static constexpr int kCells = kChainCells ? D * G::kBlock : 1;
 };
 
 // BOUND: the upstream gradient is zero on every top-level word that has a letter below BOUND after the
@@ -979,7 +986,8 @@ __device__ __forceinline__ void dense_backward_body(
     const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
     const int pu,  // prefix of the thread
     T (&sdx)[BackwardShape<T, D, N, P>::kStage],
-    T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow]) {
+    T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
+    T (&cells)[BackwardShape<T, D, N, P>::kCells]) {
     using G = Geometry<D, N, P>;
     using BS = BackwardShape<T, D, N, P>;
     constexpr int KS = N - P;
@@ -991,6 +999,13 @@ __device__ __forceinline__ void dense_backward_body(
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
+    // chain terms through LDS (see BackwardShape): the lane's cells start at zero
+    constexpr bool kCellChain = BS::kChainCells && !(sizeof(T) == 4 && P * D <= 24);
+    T *my_cells = cells + (BS::kChainCells ? (int)threadIdx.x : 0);  // cell of letter k: my_cells[k * G::kBlock]
+    if constexpr (kCellChain) {
+#pragma unroll
+        for (int k = 0; k < D; ++k) my_cells[k * G::kBlock] = T(0);
+    }
 
     const int64_t unit = blockIdx.x;
     const int64_t row = unit / chunks;
@@ -1030,6 +1045,7 @@ __device__ __forceinline__ void dense_backward_body(
             for (int k = 0; k < D; ++k) onehot[j][k] = (u[j] == k) ? T(1) : T(0);
     }
 
+
     const int64_t len = end - begin;
     const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
     for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
@@ -1062,9 +1078,19 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int j = 0; j < P; ++j) {
                     if constexpr (kOneHot) v = fmad<T>(onehot[j][k], gpre[j], v);
-                    else v += (u[j] == k) ? gpre[j] : T(0);
+                    else if constexpr (!BS::kChainCells) v += (u[j] == k) ? gpre[j] : T(0);
                 }
                 tot[k] = v;
+            }
+            if constexpr (BS::kChainCells && !kOneHot) {
+                // LDS adds, because two positions of the prefix may carry the same letter; no other lane touches
+                // these cells, and the ones just used are cleared again for the next increment
+#pragma unroll
+                for (int j = 0; j < P; ++j) atomicAdd(&my_cells[u[j] * G::kBlock], gpre[j]);
+#pragma unroll
+                for (int k = 0; k < D; ++k) tot[k] += my_cells[k * G::kBlock];
+#pragma unroll
+                for (int j = 0; j < P; ++j) my_cells[u[j] * G::kBlock] = T(0);
             }
             if constexpr (kParts == 4 && D <= 8) {
                 // all letters in one pass of exchanges (the alphabet padded to a power of two with zeros);
@@ -1158,16 +1184,17 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx[BS::kStage];
     __shared__ T sg[BS::kSums][BS::kSumRow];
+    __shared__ T cells[BS::kCells];
     if constexpr (BOUNDED) {
         const int pu = LetterBounds<D, P>::prefix_of_thread((int)threadIdx.x);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value>(
-                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, sdx, sg);
+                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, sdx, sg, cells);
         });
     } else {
         dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0>(path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape,
-                                                                chunks, grad_path, (int)threadIdx.x, sdx, sg);
+                                                                chunks, grad_path, (int)threadIdx.x, sdx, sg, cells);
     }
 }
 
