@@ -78,9 +78,12 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
  * reference, whose backward receives the path and the signature only and recomputes what it needs).
  * On long paths the register-tiled kernels cut every row into time chunks; the forward can write the
  * signature of each chunk below the top level into `chunks`, and a backward that is given the same buffer
- * skips the launch that would recompute them.  pathsig_sig_chunks_bytes() returns the size of that buffer
- * for a call, or 0 when the call has nothing to hand over (then use the plain entry points).  All other
- * arguments are as above; `chunks == NULL` makes both functions identical to the plain ones.
+ * skips the launch that would recompute them.  The per-word kernels hand over, in the same buffer, the
+ * prefix values of the words whose prefixes are not all part of the signature (the backward otherwise
+ * rebuilds them with a forward sweep, as src/pathsig/backward/sig_backward_kernels.cu:134-157 does).
+ * pathsig_sig_chunks_bytes() returns the size of that buffer for a call, or 0 when the call has nothing to
+ * hand over (then use the plain entry points).  All other arguments are as above; `chunks == NULL` makes
+ * both functions identical to the plain ones.
  */
 size_t pathsig_sig_chunks_bytes(int dtype, int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
                                 int64_t W);

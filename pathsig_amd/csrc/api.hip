@@ -97,6 +97,16 @@ int build_plan(int64_t d, int depth, const int64_t *level_sizes, int64_t n_encod
     }
     plan->block_begin[depth + 1] = blocks;
     plan->sig_size = out;
+    int64_t keep = 0;
+    for (int k = 1; k <= depth; ++k) {
+        plan->keep_off[k] = -1;
+        if (k > 1 && !plan->from_saved[k] && plan->size[k] > 0) {
+            plan->keep_off[k] = keep;
+            keep += plan->size[k] * (k - 1);
+        }
+    }
+    plan->keep_size = keep;
+    plan->keep = nullptr;
     if (enc > 0 && !have_codes) {
         set_error("encoded_words is NULL but %lld word codes are needed", (long long)enc);
         return PATHSIG_ERR_ARGUMENT;
@@ -136,8 +146,9 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
     rc = check_grid(plan, B * shape.W);
     if (rc != PATHSIG_OK) return rc;
     const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
-    if (keep && (!dc.usable || dc.keep_bytes == 0 || keep_bytes < dc.keep_bytes)) {
-        set_error("chunk buffer: this call keeps %zu bytes, got %zu", dc.usable ? dc.keep_bytes : (size_t)0, keep_bytes);
+    const size_t keep_need = dc.usable ? dc.keep_bytes : (size_t)(B * shape.W * plan.keep_size) * sizeof(T);
+    if (keep && (keep_need == 0 || keep_bytes < keep_need)) {
+        set_error("chunk buffer: this call keeps %zu bytes, got %zu", keep_need, keep_bytes);
         return PATHSIG_ERR_ARGUMENT;
     }
     if (dc.usable) {
@@ -158,6 +169,7 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
         }
         return PATHSIG_OK;
     }
+    plan.keep = keep;  // the per-word forward leaves the prefix values its backward would recompute
     hipError_t e = launch_words_forward<T>((const T *)path, (T *)sig, shape, plan, codes, stream);
     if (e != hipSuccess) return launch_failed(e, "forward launch");
     return PATHSIG_OK;
@@ -177,10 +189,12 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     rc = check_grid(plan, B * shape.W);
     if (rc != PATHSIG_OK) return rc;
     const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
-    if (kept && (!dc.usable || dc.keep_bytes == 0 || kept_bytes < dc.keep_bytes)) {
-        set_error("chunk buffer: this call keeps %zu bytes, got %zu", dc.usable ? dc.keep_bytes : (size_t)0, kept_bytes);
+    const size_t keep_need = dc.usable ? dc.keep_bytes : (size_t)(B * shape.W * plan.keep_size) * sizeof(T);
+    if (kept && (keep_need == 0 || kept_bytes < keep_need)) {
+        set_error("chunk buffer: this call keeps %zu bytes, got %zu", keep_need, kept_bytes);
         return PATHSIG_ERR_ARGUMENT;
     }
+    plan.keep = const_cast<void *>(kept);
     const size_t inc_bytes = align_up((size_t)(B * (L - 1) * d) * sizeof(T));
     const size_t need = inc_bytes + (dc.usable ? dc.backward_workspace : 0);
     if (!workspace || workspace_bytes < need) {
@@ -295,7 +309,8 @@ size_t pathsig_sig_chunks_bytes(int dtype, int64_t B, int64_t L, int64_t d, int 
     if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
     const DenseChoice dc =
         dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
-    return dc.usable ? dc.keep_bytes : 0;
+    if (dc.usable) return dc.keep_bytes;
+    return (size_t)(B * (W > 0 ? W : 1) * plan.keep_size) * elem_size(dtype);
 }
 
 int pathsig_sig_forward(const void *path, void *sig, int dtype, int64_t B, int64_t L, int64_t d, int depth,

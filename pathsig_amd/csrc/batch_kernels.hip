@@ -61,6 +61,7 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
     const T *grow = grad_sig + row * plan.sig_size;
 
     // per word: LDS offsets of the lane's increments, chain at the right end of the window, chain adjoint
+    const bool kept_chain = DEG > 1 && !plan.from_saved[DEG] && plan.keep != nullptr && plan.keep_off[DEG] >= 0;
     int aoff[WPL][DEG];
     T p[WPL][DEG + 1], h[WPL][DEG + 1];
 #pragma unroll
@@ -88,6 +89,11 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
                 off += width;
                 width *= (uint64_t)d;
             }
+        } else if (kept_chain && have && path_ok) {
+            // the forward of this call kept the chain
+            const T *kept = (const T *)plan.keep + row * plan.keep_size + plan.keep_off[DEG] + word_idx * (DEG - 1);
+#pragma unroll
+            for (int k = 1; k < DEG; ++k) p[i][k] = kept[k - 1];
         }
     }
 
@@ -138,7 +144,7 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
         return (int)(left < tile ? left : tile);
     };
 
-    if (!plan.from_saved[DEG] && DEG > 1 && ntiles > 0) {
+    if (!plan.from_saved[DEG] && DEG > 1 && ntiles > 0 && !kept_chain) {
         // chain at the right end of the window by a forward sweep (levels < DEG)
         fetch(0, tile_steps(0));
         commit(tile_steps(0));

@@ -24,6 +24,13 @@ struct LevelPlan {
     int64_t code_off[kMaxDepth + 1];
     int64_t block_begin[kMaxDepth + 2];
     int64_t sig_size;
+    // What a forward can keep for the backward of the same call: the prefix values S(w_1..w_k), k < |w|, of
+    // the words of every level whose prefixes are not all in the saved signature (from_saved == 0), which the
+    // backward would otherwise recompute with a forward sweep.  Row layout: keep_off[level] + word * (level - 1)
+    // + (k - 1); keep_off is -1 for levels that keep nothing, keep_size the elements per row.
+    int64_t keep_off[kMaxDepth + 1];
+    int64_t keep_size;
+    void *keep;  // device buffer [rows, keep_size] of the call's element type, or nullptr (nothing kept)
 };
 
 // Geometry of one signature call.

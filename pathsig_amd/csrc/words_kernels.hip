@@ -60,7 +60,14 @@ __device__ void forward_body(const T *__restrict__ path, T *__restrict__ sig, co
             }
         }
     }
-    if (active) sig[row * plan.sig_size + plan.out_off[DEG] + word_idx] = p[DEG];
+    if (active) {
+        sig[row * plan.sig_size + plan.out_off[DEG] + word_idx] = p[DEG];
+        if (plan.keep && plan.keep_off[DEG] >= 0) {
+            T *kept = (T *)plan.keep + row * plan.keep_size + plan.keep_off[DEG] + word_idx * (DEG - 1);
+#pragma unroll
+            for (int k = 1; k < DEG; ++k) kept[k - 1] = p[k];
+        }
+    }
 }
 
 template <typename T, int MAXDEG>
@@ -169,6 +176,13 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
                 off += width;
                 width *= (uint64_t)d;
             }
+        }
+    } else if (DEG > 1 && plan.keep && plan.keep_off[DEG] >= 0) {
+        // the forward of this call kept the chain
+        if (active) {
+            const T *kept = (const T *)plan.keep + row * plan.keep_size + plan.keep_off[DEG] + word_idx * (DEG - 1);
+#pragma unroll
+            for (int k = 1; k < DEG; ++k) p[k] = kept[k - 1];
         }
     } else if (DEG > 1) {
         for (int64_t t0 = 0; t0 < span.steps; t0 += tile) {

@@ -672,11 +672,14 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dt
 # hand-over of the time-chunk signatures from the forward to the backward of one call
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-@pytest.mark.parametrize("case", ["dense", "windows", "lyndon", "not_chunked", "per_word"])
+@pytest.mark.parametrize("case", ["dense", "windows", "lyndon", "not_chunked", "per_word", "words_few_paths",
+                                  "words_many_paths", "words_windows"])
 def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, case):
     """`compute_signature_keep` / `signature_backward_kept` (what the modules use when a gradient is wanted)
-    against the reference's pair `compute_signature` / `signature_backward`: same signature, same dL/dpath,
-    whether or not the call is time-chunked (the chunk buffer is empty when it is not)."""
+    against the reference's pair `compute_signature` / `signature_backward`: same signature, same dL/dpath.
+    Kept are the time-chunk signatures of the register-tiled kernels, or, on the per-word kernels, the prefix
+    values of the words whose prefixes are not in the saved signature (both backward kernels read them: lanes
+    on words for a few paths, lanes on paths for a dozen and more); the buffer is empty when neither applies."""
     import ctypes
     from pathsig_amd import _load
     depth, kw, chunked = 4, {}, True
@@ -693,8 +696,15 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, cas
         monkeypatch.setenv("PATHSIG_CHUNKS", "3")
     elif case == "not_chunked":
         d, B, L, chunked = 4, 3000, 20, False
+    elif case == "per_word":
+        d, B, L, chunked = 5, 3, 40, False          # no register-tiled shape for d = 5: per-word kernels, all dense
     else:
-        d, B, L, chunked = 5, 3, 40, False          # no register-tiled shape for d = 5: per-word kernels
+        d, depth, L = 5, 5, 60
+        B = 3 if case == "words_few_paths" else 20
+        words = random_word_set(d, 1, depth, 70, seed=403)
+        kw["projection"] = ps.projections.words(words, depth=depth, path_dim=d)
+        if case == "words_windows":
+            kw["windows"] = [(0, 60), (5, 31), (20, 21), (9, 9)]
     path = brownian_path(B, L, d, seed=401) * 1.5
     x = path.to(dtype).to(DEV)
     wins = kw.get("windows")
