@@ -159,7 +159,9 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
                     T dl[DEG];
 #pragma unroll
                     for (int k = 0; k < DEG; ++k) dl[k] = dxr[aoff[i][k]];
-                    chain_step<T, DEG, DEG - 1>(p[i], dl, T(1));
+                    T dq[DEG][DEG];
+                    scale_letters<T, DEG>(dl, dq);
+                    chain_step<T, DEG, DEG - 1, true>(p[i], dq);
                 }
             }
             lds_barrier();
@@ -186,8 +188,10 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
 #pragma unroll
                 for (int k = 0; k < DEG; ++k) dl[k] = dxr[aoff[i][k]];
                 // S_t = S_{t+1} (x) exp(-dx_t) on the chain (levels < DEG are all the adjoint needs)
-                chain_step<T, DEG, DEG - 1>(p[i], dl, T(-1));
-                chain_step_adjoint<T, DEG>(p[i], h[i], dl, gl);
+                T dq[DEG][DEG];
+                scale_letters<T, DEG>(dl, dq);
+                chain_step<T, DEG, DEG - 1, false>(p[i], dq);
+                chain_step_adjoint<T, DEG>(p[i], h[i], dl, dq, gl);
                 // cells of this lane only, so no atomics; two entries may share a cell (same letter), which
                 // keeps the read-add-writes in program order
 #pragma unroll

@@ -52,18 +52,32 @@ __device__ __forceinline__ void decode_letters(uint64_t code, uint64_t d, int (&
     }
 }
 
-// one forward Horner/Chen step on the chain p[0..TOP]; sign = +1 forward, -1 roll-back
-template <typename T, int DEG, int TOP>
-__device__ __forceinline__ void chain_step(T (&p)[DEG + 1], const T (&dl)[DEG], T sign) {
+// The letters of a word's step at every scale the chain asks for: dq[j][q - 1] = dl[j] / q, q <= DEG - j
+// (position j + 1 is divided by m - j for target level m).  With them every chain node is one FMA, as in the
+// register-tiled kernels, instead of an FMA and two multiplies.
+template <typename T, int DEG>
+__device__ __forceinline__ void scale_letters(const T (&dl)[DEG], T (&dq)[DEG][DEG]) {
+#pragma unroll
+    for (int j = 0; j < DEG; ++j) {
+        dq[j][0] = dl[j];
+#pragma unroll
+        for (int q = 2; q <= DEG - j; ++q) dq[j][q - 1] = dl[j] * Recip<T>::of(q);
+    }
+}
+
+// one forward Horner/Chen step on the chain p[0..TOP]; FORWARD = false rolls the step back (increment negated)
+template <typename T, int DEG, int TOP, bool FORWARD>
+__device__ __forceinline__ void chain_step(T (&p)[DEG + 1], const T (&dq)[DEG][DEG]) {
 #pragma unroll
     for (int m = TOP; m >= 1; --m) {
-        T s = sign * Recip<T>::of(m);
+        T tmp = T(1);
 #pragma unroll
         for (int j = 1; j < m; ++j) {
-            const T tmp = fma_t<T>(s, dl[j - 1], p[j]);
-            s = sign * tmp * Recip<T>::of(m - j);
+            const T inc = FORWARD ? dq[j - 1][m - j] : -dq[j - 1][m - j];  // dl[j - 1] / (m - j + 1)
+            tmp = j == 1 ? p[1] + inc : fma_t<T>(tmp, inc, p[j]);
         }
-        p[m] = fma_t<T>(s, dl[m - 1], p[m]);
+        const T inc = FORWARD ? dq[m - 1][0] : -dq[m - 1][0];
+        p[m] = m == 1 ? p[1] + inc : fma_t<T>(tmp, inc, p[m]);
     }
 }
 
@@ -72,24 +86,24 @@ __device__ __forceinline__ void chain_step(T (&p)[DEG + 1], const T (&dl)[DEG], 
 // step's dL/d(dl[k]).  Targets ascend, so h[m] is still the adjoint after the step when target m reads it.
 template <typename T, int DEG>
 __device__ __forceinline__ void chain_step_adjoint(const T (&p)[DEG + 1], T (&h)[DEG + 1], const T (&dl)[DEG],
-                                                   T (&gl)[DEG]) {
+                                                   const T (&dq)[DEG][DEG], T (&gl)[DEG]) {
 #pragma unroll
     for (int k = 0; k < DEG; ++k) gl[k] = T(0);
 #pragma unroll
     for (int m = 1; m <= DEG; ++m) {
-        T s[DEG + 1];
-        s[1] = Recip<T>::of(m);
+        // t[j] = Horner value after position j for target m (t[0] = 1)
+        T t[DEG + 1];
+        t[0] = T(1);
 #pragma unroll
-        for (int j = 1; j < m; ++j) {
-            const T tmp = fma_t<T>(s[j], dl[j - 1], p[j]);
-            s[j + 1] = tmp * Recip<T>::of(m - j);
-        }
+        for (int j = 1; j < m; ++j) t[j] = j == 1 ? p[1] + dq[0][m - 1] : fma_t<T>(t[j - 1], dq[j - 1][m - j], p[j]);
         T gt = h[m];
 #pragma unroll
         for (int j = m; j >= 1; --j) {
-            gl[j - 1] = fma_t<T>(gt, s[j], gl[j - 1]);
+            // node j: value p[j] + t[j - 1] * dl[j - 1] / q with q = m - j + 1
+            const T gts = j == m ? gt : gt * Recip<T>::of(m - j + 1);
+            gl[j - 1] = j == 1 ? gl[0] + gts : fma_t<T>(gts, t[j - 1], gl[j - 1]);
             if (j > 1) {
-                gt = gt * dl[j - 1] * Recip<T>::of(m - j + 1);
+                gt = gts * dl[j - 1];
                 h[j - 1] += gt;
             }
         }

@@ -56,7 +56,9 @@ __device__ void forward_body(const T *__restrict__ path, T *__restrict__ sig, co
                 T dl[DEG];
 #pragma unroll
                 for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
-                chain_step<T, DEG, DEG>(p, dl, T(1));
+                T dq[DEG][DEG];
+                scale_letters<T, DEG>(dl, dq);
+                chain_step<T, DEG, DEG, true>(p, dq);
             }
         }
     }
@@ -196,7 +198,9 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
                 T dl[DEG];
 #pragma unroll
                 for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
-                chain_step<T, DEG, DEG - 1>(p, dl, T(1));
+                T dq[DEG][DEG];
+                scale_letters<T, DEG>(dl, dq);
+                chain_step<T, DEG, DEG - 1, true>(p, dq);
             }
         }
     }
@@ -225,9 +229,11 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
 #pragma unroll
             for (int k = 0; k < DEG; ++k) dl[k] = dxr[l[k]];
             // S_t = S_{t+1} (x) exp(-dx_t) on the chain (levels < DEG are all the adjoint needs)
-            chain_step<T, DEG, DEG - 1>(p, dl, T(-1));
+            T dq[DEG][DEG];
+            scale_letters<T, DEG>(dl, dq);
+            chain_step<T, DEG, DEG - 1, false>(p, dq);
             T gl[DEG];
-            chain_step_adjoint<T, DEG>(p, h, dl, gl);
+            chain_step_adjoint<T, DEG>(p, h, dl, dq, gl);
             if (sorted) {
                 T *val = sval + (tt & 1) * (DEG * kBwdBlock);  // two buffers: one barrier per step is enough
 #pragma unroll
