@@ -11,6 +11,7 @@ import ctypes
 import os
 import pathlib
 import threading
+import warnings
 
 import torch
 
@@ -110,6 +111,11 @@ def load_torch_ops() -> bool:
         if os.environ.get("PATHSIG_PYTHON_OPS") or not path.is_file():
             _torch_ops_loaded = False
         else:
-            torch.ops.load_library(str(path))
-            _torch_ops_loaded = True
+            try:
+                torch.ops.load_library(str(path))
+                _torch_ops_loaded = True
+            except OSError as exc:  # built against another torch or an older libpathsig_hip.so
+                warnings.warn(f"{path} could not be loaded ({exc}); registering the operators from Python instead. "
+                              "Rebuild it with `python pathsig_amd/build_ext.py`.", RuntimeWarning)
+                _torch_ops_loaded = False
     return _torch_ops_loaded
