@@ -302,6 +302,8 @@ def test_sig_to_logsig_cache_layout(ps):
     (5, 2, [24, 0, 7]),
     (4, 5, "lyndon"),
     (7, 3, []),                        # empty top level
+    (8, 5, "lyndon"),                  # the size of the benchmark configuration
+    (9, 5, None),                      # odd alphabet, dense top level of 59049 words
 ])
 def test_logsig_adjoint_both_forms(ps, monkeypatch, form, dtype, d, depth, top):
     """The adjoint op against the checker, in its gather form and (forced) in its scatter form."""
