@@ -103,8 +103,11 @@ int pathsig_sig_backward_kept(const void *path, const void *sig, const void *gra
  * is dense).  Replaces sig_to_logsig (src/pathsig/forward/sig_launch.cu:230-339, op
  * `pathsig::sig_to_logsig`, src/pathsig/bindings.cpp:39-49).
  *   sig [rows, S] -> logsig [rows, S] and the power cache P [rows, S * depth] with
- *   P[idx * depth + (m - 1)] = level-|w| part of (S - 1)^(x)m at word idx, 0 for m > |w|.
- * Every element of logsig and P is written.
+ *   P[idx * depth + (m - 1)] = level-|w| part of (S - 1)^(x)m at word idx, 0 for m > |w|
+ *   (the layout and contents of src/pathsig/forward/sig_kernels.cu:184,215-216,237).
+ * Every element of logsig and P is written.  The values of logsig do not come from summing the powers in P
+ * (that alternating sum loses most digits of fp32 on long or deep inputs) but from inverting the exponential
+ * series with powers of the log-signature itself; P is filled by a second pass for callers that read it.
  */
 int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, int64_t rows, int64_t d, int depth,
                            int64_t top_size, const int64_t *top_words, void *stream);
@@ -113,12 +116,41 @@ int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, in
  * Adjoint of the above: dL/dsig from dL/dlogsig.  Replaces logsig_backward
  * (src/pathsig/backward/sig_backward_launch.cu:307-460, op `pathsig::logsig_backward`,
  * src/pathsig/bindings.cpp:52-63).
- *   sig, grad_logsig [rows, S], P [rows, S * depth] -> grad_sig [rows, S].
+ *   sig, grad_logsig [rows, S] -> grad_sig [rows, S].
+ * P is accepted for the reference's argument list and not read (it may be NULL): the adjoint rebuilds the
+ * log-signature and the cache it needs from sig inside `workspace`.
  */
 size_t pathsig_logsig_backward_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size);
 int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_logsig, void *grad_sig, int dtype,
                             int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                             void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The same pair with a hand-over from the forward to the backward (no counterpart in the reference).  The
+ * forward writes, instead of P, the cache its own adjoint reads: cache [rows, S * depth] with
+ * cache[idx * depth + (k - 1)] = level-|w| part of (log S)^(x)k at word idx (entry 0 is the log-signature
+ * itself), 0 for k > |w|.  The backward takes that cache and the log-signature and skips rebuilding them.
+ */
+int pathsig_logsig_forward_keep(const void *sig, void *logsig, void *cache, int dtype, int64_t rows, int64_t d,
+                                int depth, int64_t top_size, const int64_t *top_words, void *stream);
+size_t pathsig_logsig_backward_kept_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size);
+int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const void *grad_logsig, void *grad_sig,
+                                 int dtype, int64_t rows, int64_t d, int depth, int64_t top_size,
+                                 const int64_t *top_words, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Tuning switches (no counterpart in the reference, whose two heuristics are hard-coded:
+ * src/pathsig/forward/sig_launch.cu:23-27, src/pathsig/backward/sig_backward_launch.cu:171).  They are process
+ * wide and meant for tests and measurements; the defaults need no call.  Initial values come from the environment
+ * variables named below, which are read once, when the first call of the process needs them.
+ *   "chunks"          forced number of time chunks per row of the register-tiled kernels, 0 = chosen per call
+ *                     (PATHSIG_CHUNKS)
+ *   "letter_bounds"   1 = embedded projections leave out unwanted top-level words (PATHSIG_NO_LETTER_BOUNDS sets 0)
+ *   "logsig_scatter"  1 = the log-signature adjoint always takes its scatter form (PATHSIG_LOGSIG_SCATTER=1)
+ *   "batch_tile"      cap on the increments per tile of the lanes-on-paths backward, 0 = none (PATHSIG_BATCH_TILE)
+ * Returns PATHSIG_ERR_ARGUMENT for an unknown name or a value out of range.
+ */
+int pathsig_set_option(const char *name, int64_t value);
 
 /*
  * Measurement hook (no counterpart in the reference).  While enabled, every signature backward call brackets

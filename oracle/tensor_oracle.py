@@ -15,8 +15,10 @@ dense level-tensor form so that it can run on a CPU in fp64 and be differentiate
                        (`forward/sig_launch.cu:171-206`, `tests/test_projections.py:13-37`);
 * `tensor_log_levels`  log(1 + X) = sum_m (-1)^(m+1)/m X^(x)m with P_m = P_{m-1} (x) X
                        (`sig_kernels.cu:221-240`);
-* `hybrid_logsig`      logsig and the P cache in the "dense below the top level" layout
-                       (`src/pathsig/modules.py:98-135`, `sig_kernels.cu:184,215-216`).
+* `sig_to_logsig`      logsig and the P cache in the "dense below the top level" layout
+                       (`src/pathsig/modules.py:98-135`, `sig_kernels.cu:184,215-216`);
+* `logsig_power_cache` tensor powers of the log-signature in the same layout (what the keeping forward of the
+                       HIP library hands to its adjoint; not in the reference).
 
 Pinned by tests/test_oracle_math.py (closed forms, brute-force iterated sums, Chen, shuffle
 products, exp/log round trip, Lie property, finite differences) and cross-checked against the
@@ -167,11 +169,38 @@ def tensor_log_levels(S: List[torch.Tensor], depth: int) -> List[torch.Tensor]:
     return out
 
 
-def logsignature(path: torch.Tensor, depth: int, windows=None) -> torch.Tensor:
-    """Dense log-signature (no projection), same layout as the signature."""
+def tensor_log_levels_inverse_exp(S: List[torch.Tensor], depth: int) -> List[torch.Tensor]:
+    """The same logarithm from exp(L) = S, level by level:  L_n = S_n - sum_{k=2}^{n} (L^(x)k)_n / k!  (the k-th
+    power at level n only involves L_1 .. L_{n-1}).
+
+    Not the reference's formula (that is `tensor_log_levels`), but the same function of S, and the one to check
+    against where the alternating series is ill conditioned: the powers of X = S - 1 grow like exp|x| and cancel,
+    which costs the series about log10(max|X^(x)m|) digits even in fp64 (1e-11 at depth 12), while the powers of
+    L stay small and come with 1/k!.  Pinned by exp(L) = S with an independent exponential, by agreement with the
+    series where that is well conditioned, and against the series summed in extended precision where it is not
+    (tests/test_oracle_math.py)."""
+    L: List[torch.Tensor] = []
+    for n in range(1, depth + 1):
+        acc = S[n - 1]
+        if n >= 2:
+            known = L + [torch.zeros_like(S[k - 1]) for k in range(n, depth + 1)]
+            power = known
+            fact = 1.0
+            for k in range(2, n + 1):
+                power = tensor_product_levels(power, known, n, a0=0.0, b0=0.0)
+                fact *= k
+                acc = acc - power[n - 1] / fact
+        L.append(acc)
+    return L
+
+
+def logsignature(path: torch.Tensor, depth: int, windows=None, method: str = "series") -> torch.Tensor:
+    """Dense log-signature (no projection), same layout as the signature.  method: "series" (the reference's
+    alternating series) or "inverse_exp" (see `tensor_log_levels_inverse_exp`)."""
     d = path.shape[2]
     sig = windowed(path, depth, windows) if windows is not None else signature(path, depth)
-    return torch.cat(tensor_log_levels(split_levels(sig, d, depth), depth), dim=-1)
+    log_fn = tensor_log_levels if method == "series" else tensor_log_levels_inverse_exp
+    return torch.cat(log_fn(split_levels(sig, d, depth), depth), dim=-1)
 
 
 def hybrid_columns(d: int, depth: int, top_size: int, top_codes: Optional[Sequence[int]]) -> List[int]:
@@ -213,6 +242,29 @@ def sig_to_logsig(sig_hybrid: torch.Tensor, depth: int, d: int, top_size: Option
     Pm[0] = Pm[0] + top_only
     P_arr = torch.stack(Pm, dim=-1).reshape(*lead, -1)
     return logsig, P_arr
+
+
+def logsig_power_cache(logsig_hybrid: torch.Tensor, depth: int, d: int, top_size: Optional[int] = None,
+                       top_codes: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Cache of the keeping forward (`pathsig_logsig_forward_keep`; no counterpart in the reference): with
+    L = log S, cache[..., idx * depth + (k - 1)] = level-|w| part of L^(x)k at word idx (entry 0 is L itself),
+    zero for k above the word's length.  Built here from plain truncated tensor products of L."""
+    offs = dense_level_offsets(d, depth)
+    if top_size is None:
+        top_size = d ** depth
+    cols = hybrid_columns(d, depth, top_size, top_codes)
+    lead = logsig_hybrid.shape[:-1]
+    low = offs[depth]
+    # the top level of L enters no product that stays within `depth` letters
+    dense = torch.cat([logsig_hybrid[..., :low], torch.zeros(*lead, d ** depth, dtype=logsig_hybrid.dtype)], dim=-1)
+    L = split_levels(dense, d, depth)
+    powers = [L]
+    for _ in range(2, depth + 1):
+        powers.append(tensor_product_levels(powers[-1], L, depth, a0=0.0, b0=0.0))
+    colt = torch.tensor(cols, dtype=torch.int64)
+    Q = [torch.cat(pw, dim=-1).index_select(-1, colt) for pw in powers]
+    Q[0] = logsig_hybrid
+    return torch.stack(Q, dim=-1).reshape(*lead, -1)
 
 
 # ----------------------------------------------------------------------------------------------

@@ -8,15 +8,13 @@ There is no fallback: if the library is missing, importing the package fails.
 from __future__ import annotations
 
 import ctypes
-import os
 import pathlib
 import threading
-import warnings
 
 import torch
 
 _LIB_NAME = "libpathsig_hip.so"
-_ABI_VERSION = 2
+_ABI_VERSION = 3
 _lock = threading.Lock()
 _lib: ctypes.CDLL | None = None
 
@@ -32,6 +30,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pathsig_last_error.restype = ctypes.c_char_p
     lib.pathsig_last_error.argtypes = []
 
+    lib.pathsig_set_option.restype = _INT
+    lib.pathsig_set_option.argtypes = [ctypes.c_char_p, _I64]
     lib.pathsig_profile_enable.restype = _INT
     lib.pathsig_profile_enable.argtypes = [_INT]
     lib.pathsig_profile_sweep_ms.restype = ctypes.c_float
@@ -62,6 +62,13 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pathsig_logsig_backward.restype = _INT
     lib.pathsig_logsig_backward.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _I64, _PTR, _PTR, _SIZE,
                                             _PTR]
+    lib.pathsig_logsig_forward_keep.restype = _INT
+    lib.pathsig_logsig_forward_keep.argtypes = [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _I64, _PTR, _PTR]
+    lib.pathsig_logsig_backward_kept_workspace.restype = _SIZE
+    lib.pathsig_logsig_backward_kept_workspace.argtypes = [_INT, _I64, _I64, _INT, _I64]
+    lib.pathsig_logsig_backward_kept.restype = _INT
+    lib.pathsig_logsig_backward_kept.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _I64, _PTR, _PTR,
+                                                 _SIZE, _PTR]
 
 
 def library_path() -> pathlib.Path:
@@ -96,26 +103,32 @@ def lib() -> ctypes.CDLL:
 
 
 _TORCH_LIB_NAME = "libpathsig_torch.so"
-_torch_ops_loaded: bool | None = None
+_torch_ops_loaded = False
 
 
-def load_torch_ops() -> bool:
-    """Loads the C++ registration of the operators (schemas, device implementations, autograd) if it is built.
+def load_torch_ops() -> None:
+    """Loads the C++ registration of the operators (schemas, device implementations, autograd nodes).
 
-    Returns False when it is absent or `PATHSIG_PYTHON_OPS=1` asks for the registration from Python; both
-    run the same kernels of libpathsig_hip.so, the C++ one without the interpreter's overhead per call."""
+    There is no second registration: a missing or stale library is an error."""
     global _torch_ops_loaded
-    if _torch_ops_loaded is None:
-        ensure_loaded()
-        path = pathlib.Path(__file__).resolve().parent / _TORCH_LIB_NAME
-        if os.environ.get("PATHSIG_PYTHON_OPS") or not path.is_file():
-            _torch_ops_loaded = False
-        else:
-            try:
-                torch.ops.load_library(str(path))
-                _torch_ops_loaded = True
-            except OSError as exc:  # built against another torch or an older libpathsig_hip.so
-                warnings.warn(f"{path} could not be loaded ({exc}); registering the operators from Python instead. "
-                              "Rebuild it with `python pathsig_amd/build_ext.py`.", RuntimeWarning)
-                _torch_ops_loaded = False
-    return _torch_ops_loaded
+    if _torch_ops_loaded:
+        return
+    ensure_loaded()
+    path = pathlib.Path(__file__).resolve().parent / _TORCH_LIB_NAME
+    if not path.is_file():
+        raise RuntimeError(
+            f"Could not find the operator library {path}. Build it with `python pathsig_amd/build_ext.py` "
+            "(needs g++ and the torch headers).")
+    try:
+        torch.ops.load_library(str(path))
+    except OSError as exc:  # built against another torch or an older libpathsig_hip.so
+        raise RuntimeError(f"{path} could not be loaded ({exc}); rebuild it with "
+                           "`python pathsig_amd/build_ext.py`.") from exc
+    _torch_ops_loaded = True
+
+
+def set_option(name: str, value: int) -> None:
+    """Process-wide tuning switch of the kernel library (see `pathsig_set_option` in include/pathsig_hip.h)."""
+    rc = lib().pathsig_set_option(name.encode(), int(value))
+    if rc != 0:
+        raise ValueError(lib().pathsig_last_error().decode("utf-8", "replace"))

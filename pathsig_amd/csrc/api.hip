@@ -1,6 +1,8 @@
 // extern "C" entry points of libpathsig_hip.so: argument checks, level plans, kernel selection.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.hpp"
@@ -17,6 +19,37 @@ void set_error(const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
+}
+
+namespace {
+int64_t env_int(const char *name, int64_t fallback) {
+    const char *v = getenv(name);
+    return (v && *v) ? atoll(v) : fallback;
+}
+
+// Plain integers behind relaxed atomics: a setter on one thread and a call on another see whole values.
+struct OptionCells {
+    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile;
+    OptionCells()
+        : chunks(env_int("PATHSIG_CHUNKS", 0)),
+          letter_bounds(getenv("PATHSIG_NO_LETTER_BOUNDS") ? 0 : 1),
+          logsig_scatter(env_int("PATHSIG_LOGSIG_SCATTER", 0) == 1 ? 1 : 0),
+          batch_tile(env_int("PATHSIG_BATCH_TILE", 0)) {}
+};
+OptionCells &option_cells() {
+    static OptionCells cells;  // the environment is read here, once
+    return cells;
+}
+}  // namespace
+
+const Options &options() {
+    thread_local Options snapshot;
+    OptionCells &c = option_cells();
+    snapshot.chunks = c.chunks.load(std::memory_order_relaxed);
+    snapshot.letter_bounds = c.letter_bounds.load(std::memory_order_relaxed);
+    snapshot.logsig_scatter = c.logsig_scatter.load(std::memory_order_relaxed);
+    snapshot.batch_tile = c.batch_tile.load(std::memory_order_relaxed);
+    return snapshot;
 }
 
 namespace {
@@ -279,7 +312,7 @@ using namespace psig;
 
 extern "C" {
 
-int pathsig_abi_version(void) { return 2; }
+int pathsig_abi_version(void) { return 3; }
 
 const char *pathsig_last_error(void) { return g_error; }
 
@@ -289,6 +322,26 @@ int pathsig_profile_enable(int on) {
 }
 
 float pathsig_profile_sweep_ms(void) { return profile_sweep_ms(); }
+
+int pathsig_set_option(const char *name, int64_t value) {
+    if (!name) {
+        set_error("option name is NULL");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    if (!strcmp(name, "chunks") && value >= 0 && value <= 1024) {
+        option_cells().chunks.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "letter_bounds") && (value == 0 || value == 1)) {
+        option_cells().letter_bounds.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "logsig_scatter") && (value == 0 || value == 1)) {
+        option_cells().logsig_scatter.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "batch_tile") && value >= 0) {
+        option_cells().batch_tile.store(value, std::memory_order_relaxed);
+    } else {
+        set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    return PATHSIG_OK;
+}
 
 size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d, int depth,
                                      const int64_t *level_sizes, int64_t W) {
@@ -375,6 +428,15 @@ int pathsig_sig_backward_kept(const void *path, const void *sig, const void *gra
         set_error("W must be >= 0");
         return PATHSIG_ERR_ARGUMENT;
     }
+    if (B > 0 && (!windows || W > 0) && (!sig || !grad_sig)) {
+        // an empty signature (every level of size zero) is the one case with nothing to read behind them
+        bool empty = level_sizes != nullptr;
+        for (int k = 1; empty && k <= depth; ++k) empty = level_sizes[k] == 0;
+        if (!empty) {
+            set_error("sig and grad_sig must not be NULL");
+            return PATHSIG_ERR_ARGUMENT;
+        }
+    }
     if (dtype == PATHSIG_F32)
         return sig_backward_t<float>(path, sig, grad_sig, grad_path, B, L, d, depth, level_sizes, encoded_words,
                                      n_encoded, windows, W, chunks, chunks_bytes, workspace, workspace_bytes,
@@ -384,47 +446,131 @@ int pathsig_sig_backward_kept(const void *path, const void *sig, const void *gra
                                   (hipStream_t)stream);
 }
 
+namespace {
+int check_logsig_call(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words) {
+    int rc = check_logsig(dtype, rows, d, depth, top_size);
+    if (rc != PATHSIG_OK) return rc;
+    if (rows > 0 && top_size != checked_pow(d, depth) && top_size > 0 && !top_words) {
+        set_error("top_words is NULL but the top level is not dense");
+        return PATHSIG_ERR_ARGUMENT;
+    }
+    return PATHSIG_OK;
+}
+
+// columns of the hybrid layout
+int64_t hybrid_size(int64_t d, int depth, int64_t top_size) {
+    int64_t lower = 0, width = 1;
+    for (int k = 1; k < depth; ++k) {
+        width *= d;
+        lower += width;
+    }
+    return lower + top_size;
+}
+
+int logsig_forward_any(const void *sig, void *logsig, void *cache, void *powers, int dtype, int64_t rows, int64_t d,
+                       int depth, int64_t top_size, const int64_t *top_words, hipStream_t stream) {
+    hipError_t e;
+    if (dtype == PATHSIG_F32)
+        e = launch_logsig_forward<float>((const float *)sig, (float *)logsig, (float *)cache, (float *)powers, rows, d,
+                                         depth, top_size, top_words, stream);
+    else
+        e = launch_logsig_forward<double>((const double *)sig, (double *)logsig, (double *)cache, (double *)powers, rows,
+                                          d, depth, top_size, top_words, stream);
+    if (e != hipSuccess) return launch_failed(e, "logsig forward launch");
+    return PATHSIG_OK;
+}
+
+int logsig_backward_any(const void *logsig, const void *cache, const void *grad_logsig, void *grad_sig, int dtype,
+                        int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words, void *workspace,
+                        hipStream_t stream) {
+    hipError_t e;
+    if (dtype == PATHSIG_F32)
+        e = launch_logsig_backward<float>((const float *)logsig, (const float *)cache, (const float *)grad_logsig,
+                                          (float *)grad_sig, (float *)workspace, rows, d, depth, top_size, top_words,
+                                          stream);
+    else
+        e = launch_logsig_backward<double>((const double *)logsig, (const double *)cache, (const double *)grad_logsig,
+                                           (double *)grad_sig, (double *)workspace, rows, d, depth, top_size, top_words,
+                                           stream);
+    if (e != hipSuccess) return launch_failed(e, "logsig backward launch");
+    return PATHSIG_OK;
+}
+}  // namespace
+
 int pathsig_logsig_forward(const void *sig, void *logsig, void *P, int dtype, int64_t rows, int64_t d, int depth,
                            int64_t top_size, const int64_t *top_words, void *stream) {
-    int rc = check_logsig(dtype, rows, d, depth, top_size);
+    int rc = check_logsig_call(dtype, rows, d, depth, top_size, top_words);
     if (rc != PATHSIG_OK) return rc;
     if (rows == 0) return PATHSIG_OK;
     if (!sig || !logsig || !P) {
         set_error("sig, logsig and P must not be NULL");
         return PATHSIG_ERR_ARGUMENT;
     }
-    if (top_size != checked_pow(d, depth) && top_size > 0 && !top_words) {
-        set_error("top_words is NULL but the top level is not dense");
+    // P first serves as the cache of the pass that computes the values, then receives the powers
+    return logsig_forward_any(sig, logsig, P, P, dtype, rows, d, depth, top_size, top_words, (hipStream_t)stream);
+}
+
+int pathsig_logsig_forward_keep(const void *sig, void *logsig, void *cache, int dtype, int64_t rows, int64_t d,
+                                int depth, int64_t top_size, const int64_t *top_words, void *stream) {
+    int rc = check_logsig_call(dtype, rows, d, depth, top_size, top_words);
+    if (rc != PATHSIG_OK) return rc;
+    if (rows == 0) return PATHSIG_OK;
+    if (!sig || !logsig || !cache) {
+        set_error("sig, logsig and cache must not be NULL");
         return PATHSIG_ERR_ARGUMENT;
     }
-    hipError_t e;
-    if (dtype == PATHSIG_F32)
-        e = launch_logsig_forward<float>((const float *)sig, (float *)logsig, (float *)P, rows, d, depth, top_size,
-                                         top_words, (hipStream_t)stream);
-    else
-        e = launch_logsig_forward<double>((const double *)sig, (double *)logsig, (double *)P, rows, d, depth, top_size,
-                                          top_words, (hipStream_t)stream);
-    if (e != hipSuccess) return launch_failed(e, "logsig forward launch");
-    return PATHSIG_OK;
+    return logsig_forward_any(sig, logsig, cache, nullptr, dtype, rows, d, depth, top_size, top_words,
+                              (hipStream_t)stream);
+}
+
+size_t pathsig_logsig_backward_kept_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
+    if (check_logsig(dtype, rows, d, depth, top_size) != PATHSIG_OK) return 0;
+    return logsig_backward_bytes(dtype, rows, d, depth, top_size) + 256;
 }
 
 size_t pathsig_logsig_backward_workspace(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
     if (check_logsig(dtype, rows, d, depth, top_size) != PATHSIG_OK) return 0;
-    return logsig_backward_bytes(dtype, rows, d, depth, top_size) + 256;
+    // the log-signature and its cache are rebuilt in front of the adjoint's own scratch
+    const size_t S = (size_t)hybrid_size(d, depth, top_size);
+    const size_t rebuilt = align_up((size_t)rows * S * elem_size(dtype)) + align_up((size_t)rows * S * depth * elem_size(dtype));
+    return rebuilt + logsig_backward_bytes(dtype, rows, d, depth, top_size) + 256;
 }
 
 int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_logsig, void *grad_sig, int dtype,
                             int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                             void *workspace, size_t workspace_bytes, void *stream) {
-    int rc = check_logsig(dtype, rows, d, depth, top_size);
+    (void)P;  // the adjoint works from the cache of the Q form, which it rebuilds from sig
+    int rc = check_logsig_call(dtype, rows, d, depth, top_size, top_words);
     if (rc != PATHSIG_OK) return rc;
     if (rows == 0) return PATHSIG_OK;
-    if (!sig || !P || !grad_logsig || !grad_sig) {
-        set_error("sig, P, grad_logsig and grad_sig must not be NULL");
+    if (!sig || !grad_logsig || !grad_sig) {
+        set_error("sig, grad_logsig and grad_sig must not be NULL");
         return PATHSIG_ERR_ARGUMENT;
     }
-    if (top_size != checked_pow(d, depth) && top_size > 0 && !top_words) {
-        set_error("top_words is NULL but the top level is not dense");
+    const size_t S = (size_t)hybrid_size(d, depth, top_size);
+    const size_t lg_bytes = align_up((size_t)rows * S * elem_size(dtype));
+    const size_t cache_bytes = align_up((size_t)rows * S * depth * elem_size(dtype));
+    const size_t need = lg_bytes + cache_bytes + logsig_backward_bytes(dtype, rows, d, depth, top_size);
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    unsigned char *ws = (unsigned char *)workspace;
+    void *lg = ws, *cache = ws + lg_bytes, *rest = ws + lg_bytes + cache_bytes;
+    rc = logsig_forward_any(sig, lg, cache, nullptr, dtype, rows, d, depth, top_size, top_words, (hipStream_t)stream);
+    if (rc != PATHSIG_OK) return rc;
+    return logsig_backward_any(lg, cache, grad_logsig, grad_sig, dtype, rows, d, depth, top_size, top_words, rest,
+                               (hipStream_t)stream);
+}
+
+int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const void *grad_logsig, void *grad_sig,
+                                 int dtype, int64_t rows, int64_t d, int depth, int64_t top_size,
+                                 const int64_t *top_words, void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = check_logsig_call(dtype, rows, d, depth, top_size, top_words);
+    if (rc != PATHSIG_OK) return rc;
+    if (rows == 0) return PATHSIG_OK;
+    if (!logsig || !cache || !grad_logsig || !grad_sig) {
+        set_error("logsig, cache, grad_logsig and grad_sig must not be NULL");
         return PATHSIG_ERR_ARGUMENT;
     }
     const size_t need = logsig_backward_bytes(dtype, rows, d, depth, top_size);
@@ -432,17 +578,8 @@ int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_log
         set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
         return PATHSIG_ERR_WORKSPACE;
     }
-    hipError_t e;
-    if (dtype == PATHSIG_F32)
-        e = launch_logsig_backward<float>((const float *)sig, (const float *)P, (const float *)grad_logsig,
-                                          (float *)grad_sig, (float *)workspace, rows, d, depth, top_size, top_words,
-                                          (hipStream_t)stream);
-    else
-        e = launch_logsig_backward<double>((const double *)sig, (const double *)P, (const double *)grad_logsig,
-                                           (double *)grad_sig, (double *)workspace, rows, d, depth, top_size, top_words,
-                                           (hipStream_t)stream);
-    if (e != hipSuccess) return launch_failed(e, "logsig backward launch");
-    return PATHSIG_OK;
+    return logsig_backward_any(logsig, cache, grad_logsig, grad_sig, dtype, rows, d, depth, top_size, top_words,
+                               workspace, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -301,10 +301,7 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
     int64_t tile = max_block_lds() / per_step;
     if (tile > 8) tile = 8;
     if (tile * shape.d > kBatchChunks * kWave) tile = kBatchChunks * kWave / shape.d;
-    if (const char *env = getenv("PATHSIG_BATCH_TILE")) {
-        const int64_t forced = atoll(env);
-        if (forced >= 1 && forced < tile) tile = forced;
-    }
+    if (const int64_t forced = options().batch_tile; forced >= 1 && forced < tile) tile = forced;
     if (tile > shape.L - 1) tile = shape.L - 1;
     if (tile < 1) return hipErrorInvalidValue;
     const size_t lds = (size_t)(tile * per_step);

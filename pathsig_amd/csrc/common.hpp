@@ -41,6 +41,16 @@ struct SigShape {
 
 void set_error(const char *fmt, ...);
 
+// Tuning switches of the library (pathsig_set_option).  Their initial values come from the environment, read
+// once when the first call needs them; nothing on a call's path reads the environment.
+struct Options {
+    int64_t chunks;          // forced number of time chunks of the register-tiled kernels (0: chosen per call)
+    int64_t letter_bounds;   // embedded projections leave out top-level words by letter bounds (default 1)
+    int64_t logsig_scatter;  // log-signature adjoint in its scatter form even where the gather form fits (default 0)
+    int64_t batch_tile;      // cap on the increments per tile of the lanes-on-paths backward (0: no cap)
+};
+const Options &options();
+
 #if defined(__HIPCC__)
 // Wave-wide sum of one value per lane; the total is valid in lane 63 only.
 template <int CTRL, int ROW_MASK>
@@ -121,9 +131,11 @@ hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan
 template <typename T>
 hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
                                      hipStream_t stream);
+// sig -> logsig and the cache its adjoint reads; `powers`, when not null, also receives the power cache of the
+// reference (it may be the same buffer as `cache`, which it then replaces)
 template <typename T>
-hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, int64_t d, int depth, int64_t top_size,
-                                 const int64_t *top_words, hipStream_t stream);
+hipError_t launch_logsig_forward(const T *sig, T *logsig, T *cache, T *powers, int64_t rows, int64_t d, int depth,
+                                 int64_t top_size, const int64_t *top_words, hipStream_t stream);
 // workspace of the log-signature adjoint, in elements of the floating type (see logsig_kernels.hip)
 struct LogsigBackwardPlan {
     bool gather;
@@ -131,7 +143,7 @@ struct LogsigBackwardPlan {
 };
 LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, int depth, int64_t top_size);
 template <typename T>
-hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *workspace,
+hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad_logsig, T *grad_sig, T *workspace,
                                   int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                                   hipStream_t stream);
 

@@ -1496,13 +1496,10 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             dc.embed = true;
             dc.dense_bytes = pad256((size_t)rows * v.sig_size * elem);
             dc.bounded = v.bounds_ok && level_sizes[depth] > 0 && level_sizes[depth] < top_dense &&
-                         !getenv("PATHSIG_NO_LETTER_BOUNDS");
+                         options().letter_bounds != 0;
         }
         int chunks = pick_chunks(rows, v.block, L);
-        if (const char *env = getenv("PATHSIG_CHUNKS")) {
-            const int forced = atoi(env);
-            if (forced >= 1 && forced <= 1024) chunks = forced;
-        }
+        if (const int64_t forced = options().chunks; forced >= 1 && forced <= 1024) chunks = (int)forced;
         if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
         dc.variant = i;

@@ -2,18 +2,28 @@
 // a list of words).  One workgroup owns one row (one path, or one window of one path) and walks the
 // levels itself, so the whole conversion is one launch per direction.
 //
-// Forward (reference: src/pathsig/forward/sig_kernels.cu:161-241): with X = S - 1,
+// The reference (src/pathsig/forward/sig_kernels.cu:161-241) sums the series of log(1 + X), X = S - 1:
 //     P_1(w) = S(w),  P_m(w) = sum_{k=m-1}^{n-1} P_{m-1}(w_1..w_k) * S(w_{k+1}..w_n),
 //     log S(w) = sum_m (-1)^(m+1)/m * P_m(w).
-// Level n reads the P rows of the levels below it, so levels go up with a workgroup barrier between.
-// Backward (reference: src/pathsig/backward/sig_backward_kernels.cu:381-477) is the adjoint, levels
-// going down; the P adjoint of the lower levels lives in the caller's workspace.  Two forms:
-//   * gather form (used whenever a dense copy of the top-level gradient fits the workspace): with
-//     a_m(w) = dL/dP_m(w) and c_m = (-1)^(m+1)/m,
-//         a_m(w) = c_m g(w) + sum_{v, |wv| <= depth} a_{m+1}(wv) S(v),
-//         dL/dS(v) = a_1(v) + sum_{u, |uv| <= depth} sum_{m=2}^{|u|+1} a_m(uv) P_{m-1}(u),
-//     and a_m(x) = c_m g(x) for top-level words x.  Every sum over v (or u) of a fixed length is a
-//     matrix-vector product over a dense level, so each output has one owner and nothing is atomic;
+// The powers of X grow like exp|x| and cancel in the alternating sum, which costs that series most of the
+// digits of fp32 on long or deep inputs.  The values are therefore computed by inverting the exponential
+// instead, with powers of the (much smaller) log-signature L itself and the coefficients 1/k! :
+//     Q_1(w) = L(w),  Q_k(w) = sum_{j=k-1}^{n-1} Q_{k-1}(w_1..w_j) * L(w_{j+1}..w_n),
+//     L(w) = S(w) - sum_{k=2}^{n} Q_k(w) / k! .
+// Same recursion shape, same cost, same cache layout (row idx, entry k - 1); the cache of this form is what
+// the adjoint below reads.  The power cache P of the reference is still produced, by a second pass of the
+// same kernel, for the entry point that returns it.
+//
+// Backward (reference: src/pathsig/backward/sig_backward_kernels.cu:381-477, the adjoint of the P form) is
+// the adjoint of the Q form, levels going down.  With lam(w) = dLoss/dL(w), a_k(w) = dLoss/dQ_k(w), f_k = 1/k!
+// and g the upstream gradient,
+//     lam(w) = g(w) + a_1(w) + sum_{u} sum_{k=2}^{|u|+1} a_k(u w) Q_{k-1}(u),
+//     a_k(w) = -[k >= 2] f_k lam(w) + sum_{v, |wv| <= depth} a_{k+1}(w v) L(v),
+//     dLoss/dS(w) = lam(w);  for top-level words lam = g and a_k = -f_k g.
+// Two forms:
+//   * gather form (used whenever a dense copy of the top-level gradient fits the workspace): every sum over
+//     v (or u) of a fixed length is a matrix-vector product over a dense level, so each output has one owner
+//     and nothing is atomic;
 //   * scatter form (any size): every word pushes its terms to its prefixes and suffixes with atomics.
 #include <cstdlib>
 
@@ -25,12 +35,6 @@ namespace {
 
 constexpr int kLogBlock = 512;
 
-template <typename T>
-__device__ __forceinline__ T alt_coeff(int m) {
-    const T r = T(1) / T(m);
-    return (m & 1) ? r : -r;
-}
-
 struct HybridPlan {
     int depth;
     int64_t d;
@@ -41,16 +45,29 @@ struct HybridPlan {
     int top_is_list;   // top level takes its codes from top_words
 };
 
-template <typename T, int DEG>
-__device__ void logsig_forward_level(const T *__restrict__ s, T *P, T *__restrict__ lg, const HybridPlan &hp,
+// 1/k! for the exponential series
+template <typename T>
+__device__ __forceinline__ constexpr T inv_factorial(int k) {
+    T r = T(1);
+    for (int i = 2; i <= k; ++i) r /= T(i);
+    return r;
+}
+
+// One level of one row.  STABLE: C is the cache of the Q form (entry k - 1 of a row holds Q_k; entry 0 the
+// log-signature itself), the right factors are log-signature values of the levels below, read from lg, and
+// lg receives the level.  Otherwise C is the power cache P of the reference, the right factors are signature
+// values, and lg is not touched.
+template <typename T, int DEG, bool STABLE>
+__device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const HybridPlan &hp,
                                      const int64_t *__restrict__ top_words) {
     const int depth = hp.depth;
     const uint64_t d = (uint64_t)hp.d;
     const bool listed = (DEG == depth) && hp.top_is_list;
+    const T *right = STABLE ? lg : s;
     // the blocks of one row (gridDim.y of them) share the words of the level
     for (int64_t i = (int64_t)blockIdx.y * kLogBlock + threadIdx.x; i < hp.size[DEG]; i += (int64_t)gridDim.y * kLogBlock) {
         const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
-        // dense column of every proper prefix, value of every proper suffix
+        // dense column of every proper prefix, right factor of every proper suffix
         uint64_t pidx[DEG + 1];
         T sufv[DEG + 1];
         {
@@ -62,45 +79,48 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *P, T *__restric
             for (int k = 1; k < DEG; ++k) {
                 width *= d;
                 pidx[k] = lo + code / div;  // first k letters
-                sufv[k] = s[lo + code % width];  // last k letters
+                sufv[k] = right[lo + code % width];  // last k letters
                 lo += width;
                 div /= d;
             }
         }
         const uint64_t own = (uint64_t)(hp.off[DEG] + i);
         const T sw = s[own];
-        sufv[DEG] = sw;
-        T *Pw = P + own * (uint64_t)depth;
-        Pw[0] = sw;
+        T *Cw = C + own * (uint64_t)depth;
         T acc = sw;
 #pragma unroll
         for (int m = 2; m <= DEG; ++m) {
             T pv = T(0);
 #pragma unroll
-            for (int k = m - 1; k < DEG; ++k) pv += P[pidx[k] * (uint64_t)depth + (uint64_t)(m - 2)] * sufv[DEG - k];
-            acc += alt_coeff<T>(m) * pv;
-            Pw[m - 1] = pv;
+            for (int k = m - 1; k < DEG; ++k) pv += C[pidx[k] * (uint64_t)depth + (uint64_t)(m - 2)] * sufv[DEG - k];
+            if constexpr (STABLE) acc -= inv_factorial<T>(m) * pv;
+            Cw[m - 1] = pv;
         }
-        for (int m = DEG + 1; m <= depth; ++m) Pw[m - 1] = T(0);
-        lg[own] = acc;
+        for (int m = DEG + 1; m <= depth; ++m) Cw[m - 1] = T(0);
+        if constexpr (STABLE) {
+            Cw[0] = acc;
+            lg[own] = acc;
+        } else {
+            Cw[0] = sw;
+        }
     }
 }
 
 // Levels first..last of one row per blockIdx.x.  Several levels need one block per row (gridDim.y == 1: the
 // barrier between levels is a workgroup barrier); a single level may be shared by gridDim.y blocks.
-template <typename T>
-__global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__restrict__ sig, T *__restrict__ logsig,
-                                                                   T *P, HybridPlan hp,
+template <typename T, bool STABLE>
+__global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__restrict__ sig, T *logsig, T *C,
+                                                                   HybridPlan hp,
                                                                    const int64_t *__restrict__ top_words, int first,
                                                                    int last) {
     const int64_t row = blockIdx.x;
     const T *s = sig + row * hp.total;
     T *lg = logsig + row * hp.total;
-    T *Pr = P + row * hp.total * hp.depth;
+    T *Cr = C + row * hp.total * hp.depth;
     for (int deg = first; deg <= last; ++deg) {
         switch (deg) {
 #define PSIG_CASE(N) \
-    case N: logsig_forward_level<T, N>(s, Pr, lg, hp, top_words); break;
+    case N: logsig_forward_level<T, N, STABLE>(s, Cr, lg, hp, top_words); break;
             PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
             PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
 #undef PSIG_CASE
@@ -132,10 +152,18 @@ struct AdjointSink {
     __device__ __forceinline__ T read_gP(uint64_t col, int m_index) const {
         return ((int64_t)col < lds_cols) ? lds_gP[col * depth + m_index] : gP[col * depth + m_index];
     }
+    __device__ __forceinline__ T read_gs(uint64_t col) const { return ((int64_t)col < lds_cols) ? lds_gs[col] : gs[col]; }
+    __device__ __forceinline__ void set_gs(uint64_t col, T v) {
+        if ((int64_t)col < lds_cols) lds_gs[col] = v;
+        else gs[col] = v;
+    }
 };
 
+// lgrow: the log-signature row; C: the cache row of the Q form.  When a level is processed, everything the
+// longer words push to it has arrived (levels go down with a barrier between them): the accumulated gradient
+// of a word holds its suffix-type sums and entry k - 1 of its cache adjoint holds sum_v a_{k+1}(w v) L(v).
 template <typename T, int DEG>
-__device__ void logsig_backward_level(const T *__restrict__ s, const T *__restrict__ P, const T *__restrict__ gl,
+__device__ void logsig_backward_level(const T *__restrict__ lgrow, const T *__restrict__ C, const T *__restrict__ gl,
                                       AdjointSink<T> &sink, const HybridPlan &hp,
                                       const int64_t *__restrict__ top_words) {
     const int depth = hp.depth;
@@ -160,37 +188,36 @@ __device__ void logsig_backward_level(const T *__restrict__ s, const T *__restri
             }
         }
         const uint64_t own = (uint64_t)(hp.off[DEG] + i);
-        const T g = gl[own];
-        T gPv[DEG];
+        // a top-level word is nobody's prefix or suffix: nothing has been accumulated for it
+        T lam = gl[own];
+        if (!top) lam += sink.read_gP(own, 0) + sink.read_gs(own);
+        T av[DEG];
 #pragma unroll
-        for (int m = 1; m <= DEG; ++m) {
-            // a top-level word is nobody's prefix: nothing has been accumulated for it
-            const T acc = top ? T(0) : sink.read_gP(own, m - 1);
-            gPv[m - 1] = alt_coeff<T>(m) * g + acc;
-        }
-        sink.add_gs(own, gPv[0]);
+        for (int k = 2; k <= DEG; ++k) av[k - 1] = (top ? T(0) : sink.read_gP(own, k - 1)) - inv_factorial<T>(k) * lam;
+        sink.set_gs(own, lam);
 #pragma unroll
-        for (int m = 2; m <= DEG; ++m) {
+        for (int k = 2; k <= DEG; ++k) {
 #pragma unroll
-            for (int k = m - 1; k < DEG; ++k) {
-                const uint64_t pi = pidx[k], si = sidx[DEG - k];
-                sink.add_gP(pi, m - 2, gPv[m - 1] * s[si]);
-                sink.add_gs(si, gPv[m - 1] * P[pi * (uint64_t)depth + (uint64_t)(m - 2)]);
+            for (int j = k - 1; j < DEG; ++j) {
+                const uint64_t pi = pidx[j], si = sidx[DEG - j];
+                sink.add_gP(pi, k - 2, av[k - 1] * lgrow[si]);
+                sink.add_gs(si, av[k - 1] * C[pi * (uint64_t)depth + (uint64_t)(k - 2)]);
             }
         }
     }
 }
 
 template <typename T>
-__global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__restrict__ sig, const T *__restrict__ P,
+__global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__restrict__ logsig,
+                                                                    const T *__restrict__ cache,
                                                                     const T *__restrict__ grad_logsig, T *grad_sig,
                                                                     T *gradP, HybridPlan hp,
                                                                     const int64_t *__restrict__ top_words,
                                                                     int64_t lds_cols) {
     extern __shared__ __align__(16) unsigned char logsig_smem[];
     const int64_t row = blockIdx.x;
-    const T *s = sig + row * hp.total;
-    const T *Pr = P + row * hp.total * hp.depth;
+    const T *s = logsig + row * hp.total;
+    const T *Pr = cache + row * hp.total * hp.depth;
     const T *gl = grad_logsig + row * hp.total;
     AdjointSink<T> sink;
     sink.gs = grad_sig + row * hp.total;
@@ -283,12 +310,12 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
 }
 
 // Top-level part of the gather form, one block per (row, split, side): with the top-level gradient g as a
-// d^j x d^(N-j) matrix, side 0 computes R(u) = sum_v g(uv) S(v) for the prefixes u of length j, side 1
-// computes T(v) = sum_u g(uv) Q(u) for the suffixes v of length N - j, where
-// Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) comes from logsig_q_kernel.  R goes to its own workspace array, T
+// d^j x d^(N-j) matrix, side 0 computes R(u) = sum_v g(uv) L(v) for the prefixes u of length j, side 1
+// computes T(v) = sum_u g(uv) Qc(u) for the suffixes v of length N - j, where
+// Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! comes from logsig_q_kernel.  R goes to its own workspace array, T
 // initialises the gradient.
 template <typename T>
-__global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *__restrict__ sig,
+__global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *__restrict__ logsig,
                                                                       const T *__restrict__ Q_all,
                                                                       const T *__restrict__ gtop_all, T *grad_sig,
                                                                       T *R_all, HybridPlan hp, int64_t top_dense) {
@@ -297,14 +324,14 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *_
     const int64_t row = blockIdx.x;
     const int j = (int)blockIdx.y + 1, i = N - j;
     const bool suffix_side = blockIdx.z == 1;
-    const T *s = sig + row * hp.total;
+    const T *lgs = logsig + row * hp.total;
     const T *gtop = gtop_all + row * top_dense;
     int64_t wi = 1, wj = 1;
     for (int k = 0; k < i; ++k) wi *= hp.d;
     for (int k = 0; k < j; ++k) wj *= hp.d;
     if (!suffix_side) {
         T *R = R_all + row * hp.lower + hp.off[j];
-        block_matvec<T>(gtop, s + hp.off[i], MatvecShape{1, wj, wi, 1, 0, wi, 1, 0, 0, 1, 0}, red,
+        block_matvec<T>(gtop, lgs + hp.off[i], MatvecShape{1, wj, wi, 1, 0, wi, 1, 0, 0, 1, 0}, red,
                         [&](int64_t, int64_t o, T r) { R[o] = r; });
     } else {
         T *gsi = grad_sig + row * hp.total + hp.off[i];
@@ -313,9 +340,9 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *_
     }
 }
 
-// Q(u) = sum_{m=2}^{|u|+1} c_m P_{m-1}(u) for every column below the top, all rows
+// Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! for every column below the top, all rows
 template <typename T>
-__global__ void logsig_q_kernel(const T *__restrict__ P, T *__restrict__ Q_all, HybridPlan hp, int64_t rows) {
+__global__ void logsig_q_kernel(const T *__restrict__ cache, T *__restrict__ Q_all, HybridPlan hp, int64_t rows) {
     const int N = hp.depth;
     const int64_t total = rows * hp.lower;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -323,23 +350,24 @@ __global__ void logsig_q_kernel(const T *__restrict__ P, T *__restrict__ Q_all, 
         const int64_t row = idx / hp.lower, col = idx - row * hp.lower;
         int n = 1;
         while (n + 1 < N && col >= hp.off[n + 1]) ++n;
-        const T *Pc = P + (row * hp.total + col) * N;
+        const T *Cc = cache + (row * hp.total + col) * N;
         T q = T(0);
-        T sign = T(-1);
-        for (int m = 2; m <= n + 1; ++m) {
-            q += sign * Pc[m - 2] / T(m);
-            sign = -sign;
+        T f = T(1);
+        for (int k = 2; k <= n + 1; ++k) {
+            f /= T(k);
+            q -= f * Cc[k - 2];
         }
         Q_all[idx] = q;
     }
 }
 
-// Levels below the top, one block per row.  `a` ([lower columns][depth]) holds a_m: in LDS when the launch
-// provides room for it (a_in_lds; the kernel is a chain of short dependent passes over `a`, so their latency is
-// what it costs), else in the workspace.  `R` ([lower columns], workspace) are the top-level sums of
+// Levels below the top, one block per row, going down.  `a` ([lower columns][depth]) holds a_k: in LDS when the
+// launch provides room for it (a_in_lds; the kernel is a chain of short dependent passes over `a`, so their
+// latency is what it costs), else in the workspace.  `R` ([lower columns], workspace) are the top-level sums of
 // logsig_gather_top_kernel, which has also stored the top-level part of the gradient in grad_sig.
 template <typename T>
-__global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ sig, const T *__restrict__ P,
+__global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ logsig,
+                                                                  const T *__restrict__ cache,
                                                                   const T *__restrict__ grad_logsig, T *grad_sig,
                                                                   T *a_all, const T *__restrict__ R_all, HybridPlan hp,
                                                                   int a_in_lds) {
@@ -347,8 +375,8 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
     const int64_t row = blockIdx.x;
-    const T *s = sig + row * hp.total;
-    const T *Pr = P + row * hp.total * N;
+    const T *lgs = logsig + row * hp.total;
+    const T *Cr = cache + row * hp.total * N;
     const T *gl = grad_logsig + row * hp.total;
     T *gs = grad_sig + row * hp.total;
     T *a = a_in_lds ? reinterpret_cast<T *>(gather_smem) : a_all + row * hp.lower * N;
@@ -357,40 +385,50 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     width[0] = 1;
     for (int k = 1; k <= N; ++k) width[k] = width[k - 1] * hp.d;
 
-    // a_m(w) = c_m g(w) + c_{m+1} R(w) for every column below the top; the top-level columns of the
-    // gradient are a_1 = g
+    // a_k(w) starts from its top-level part, sum_v a_{k+1}(w v) L(v) = -f_{k+1} R(w); the top-level columns
+    // of the gradient are g
     for (int n = 1; n < N; ++n) {
         for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
             const int64_t col = hp.off[n] + i;
-            const T g = gl[col], r = R[col];
-            for (int m = 1; m <= N; ++m)
-                a[col * N + m - 1] = m <= n ? alt_coeff<T>(m) * g + alt_coeff<T>(m + 1) * r : T(0);
+            const T r = R[col];
+            T f = T(1);
+            for (int m = 1; m <= N; ++m) {
+                f /= T(m + 1);  // 1 / (m + 1)!
+                a[col * N + m - 1] = m <= n ? -f * r : T(0);
+            }
         }
     }
     for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) gs[hp.off[N] + i] = gl[hp.off[N] + i];
     __threadfence_block();
     __syncthreads();
 
-    // levels below the top, going down: a_m(w) += sum_v a_{m+1}(wv) S(v), all m of a level in one batch
-    for (int n = N - 2; n >= 1; --n) {
+    for (int n = N - 1; n >= 1; --n) {
         T *an = a + hp.off[n] * N;
+        T *gsn = gs + hp.off[n];
+        // a_k(w) += sum_v a_{k+1}(w v) L(v) over the levels between this one and the top, all k in one batch
         for (int i = 1; n + i < N; ++i) {
-            block_matvec<T>(a + hp.off[n + i] * N + 1, s + hp.off[i],
+            block_matvec<T>(a + hp.off[n + i] * N + 1, lgs + hp.off[i],
                             MatvecShape{n, width[n], width[i], 1, 1, width[i] * N, N, 0, 0, 1, 0}, red,
                             [&](int64_t bi, int64_t o, T r) { an[o * N + bi] += r; });
         }
-    }
-    // gradient of the lower levels: a_1(v) + sum_u sum_{m=2}^{|u|+1} a_m(uv) P_{m-1}(u)
-    for (int i = 1; i < N; ++i) {
-        T *gsi = gs + hp.off[i];
-        for (int64_t v = threadIdx.x; v < width[i]; v += kLogBlock) gsi[v] += a[(hp.off[i] + v) * N];
+        // gradient += sum_u sum_{k=2}^{|u|+1} a_k(u w) Q_{k-1}(u) over the same levels
+        for (int j = 1; n + j < N; ++j) {
+            block_matvec<T>(a + hp.off[n + j] * N + 1, Cr + hp.off[j] * N,
+                            MatvecShape{1, width[n], width[j], j, 0, N, width[n] * N, 1, 0, N, 1}, red,
+                            [&](int64_t, int64_t o, T r) { gsn[o] += r; });
+        }
+        // lam(w) = g(w) + a_1(w) + the sums above is the gradient of the word; a_k(w) -= lam(w) / k! for k >= 2
+        for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
+            const T lam = gl[hp.off[n] + i] + an[i * N] + gsn[i];
+            gsn[i] = lam;
+            T f = T(1);
+            for (int k = 2; k <= n; ++k) {
+                f /= T(k);
+                an[i * N + k - 1] -= f * lam;
+            }
+        }
         __threadfence_block();
         __syncthreads();
-        for (int j = 1; i + j < N; ++j) {
-            block_matvec<T>(a + hp.off[i + j] * N + 1, Pr + hp.off[j] * N,
-                            MatvecShape{1, width[i], width[j], j, 0, N, width[i] * N, 1, 0, N, 1}, red,
-                            [&](int64_t, int64_t o, T r) { gsi[o] += r; });
-        }
     }
 }
 
@@ -438,27 +476,40 @@ HybridPlan make_hybrid(int64_t d, int depth, int64_t top_size, const int64_t *to
 
 }  // namespace
 
-template <typename T>
-hipError_t launch_logsig_forward(const T *sig, T *logsig, T *P, int64_t rows, int64_t d, int depth, int64_t top_size,
-                                 const int64_t *top_words, hipStream_t stream) {
-    if (rows <= 0) return hipSuccess;
-    const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
-    // The top level only reads the cache rows of the levels below it: when it is large it gets a launch of its
-    // own, with its words dealt out to several blocks per row.
+namespace {
+// one pass over all levels of all rows: the top level only reads the cache rows of the levels below it, so when
+// it is large it gets a launch of its own, with its words dealt out to several blocks per row
+template <typename T, bool STABLE>
+hipError_t forward_pass(const T *sig, T *logsig, T *C, const HybridPlan &hp, int64_t rows, int64_t top_size,
+                        const int64_t *top_words, hipStream_t stream) {
+    const int depth = hp.depth;
     int64_t slices = (top_size + 4 * kLogBlock - 1) / (4 * kLogBlock);
     if (slices > 16) slices = 16;
     if (depth < 2 || slices < 2) {
-        hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig, P, hp,
-                           top_words, 1, depth);
+        hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig,
+                           logsig, C, hp, top_words, 1, depth);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig, P, hp,
-                       top_words, 1, depth - 1);
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig,
+                       C, hp, top_words, 1, depth - 1);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(logsig_forward_kernel<T>, dim3((unsigned)rows, (unsigned)slices), dim3(kLogBlock), 0, stream, sig,
-                       logsig, P, hp, top_words, depth, depth);
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows, (unsigned)slices), dim3(kLogBlock), 0,
+                       stream, sig, logsig, C, hp, top_words, depth, depth);
     return hipGetLastError();
+}
+}  // namespace
+
+// logsig and `cache` (the Q form) are always written; `powers` (the P cache of the reference), when not null,
+// is written by a second pass and may be the same buffer as `cache`, which it then replaces.
+template <typename T>
+hipError_t launch_logsig_forward(const T *sig, T *logsig, T *cache, T *powers, int64_t rows, int64_t d, int depth,
+                                 int64_t top_size, const int64_t *top_words, hipStream_t stream) {
+    if (rows <= 0) return hipSuccess;
+    const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
+    hipError_t e = forward_pass<T, true>(sig, logsig, cache, hp, rows, top_size, top_words, stream);
+    if (e != hipSuccess || powers == nullptr) return e;
+    return forward_pass<T, false>(sig, logsig, powers, hp, rows, top_size, top_words, stream);
 }
 
 // Workspace of the adjoint in elements of T: [a: rows x lower x depth][R, Q: rows x lower each][dense top gradient:
@@ -476,8 +527,7 @@ LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, in
     lp.top_elems = 0;
     lp.top_dense = width;
     lp.gather = false;
-    const char *env = getenv("PATHSIG_LOGSIG_SCATTER");
-    const bool forced_scatter = env && env[0] == '1';
+    const bool forced_scatter = options().logsig_scatter != 0;
     const bool listed = top_size != width;
     // the dense copy of the top-level gradient must stay modest: 1 GiB
     const bool fits = (double)rows * (double)width * (double)elem <= 1073741824.0;
@@ -489,8 +539,9 @@ LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, in
     return lp;
 }
 
+// logsig and cache are the outputs of launch_logsig_forward for the same signature
 template <typename T>
-hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig, T *grad_sig, T *workspace,
+hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad_logsig, T *grad_sig, T *workspace,
                                   int64_t rows, int64_t d, int depth, int64_t top_size, const int64_t *top_words,
                                   hipStream_t stream) {
     if (rows <= 0) return hipSuccess;
@@ -522,10 +573,10 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
             int64_t blocks = (rows * hp.lower + 255) / 256;
             if (blocks > 65536) blocks = 65536;
             if (blocks < 1) blocks = 1;
-            hipLaunchKernelGGL(logsig_q_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, P, Q, hp, rows);
+            hipLaunchKernelGGL(logsig_q_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, cache, Q, hp, rows);
         }
         hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2), dim3(kLogBlock), 0,
-                           stream, sig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
+                           stream, logsig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         // the adjoint of the cache goes to LDS when a block's share of it fits beside the static arrays
@@ -537,18 +588,18 @@ hipError_t launch_logsig_backward(const T *sig, const T *P, const T *grad_logsig
             if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), a_in_lds ? a_bytes : 0, stream,
-                           sig, P, grad_logsig, grad_sig, gradP, (const T *)R, hp, a_in_lds ? 1 : 0);
+                           logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp, a_in_lds ? 1 : 0);
         return hipGetLastError();
     }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
     const size_t lds_bytes = (size_t)lds_cols * (size_t)(depth + 1) * sizeof(T);
-    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), lds_bytes, stream, sig, P,
+    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), lds_bytes, stream, logsig, cache,
                        grad_logsig, grad_sig, gradP, hp, top_words, lds_cols);
     return hipGetLastError();
 }
 
 #define PSIG_INSTANTIATE(T)                                                                                       \
-    template hipError_t launch_logsig_forward<T>(const T *, T *, T *, int64_t, int64_t, int, int64_t,             \
+    template hipError_t launch_logsig_forward<T>(const T *, T *, T *, T *, int64_t, int64_t, int, int64_t,        \
                                                  const int64_t *, hipStream_t);                                   \
     template hipError_t launch_logsig_backward<T>(const T *, const T *, const T *, T *, T *, int64_t, int64_t, int, \
                                                   int64_t, const int64_t *, hipStream_t);

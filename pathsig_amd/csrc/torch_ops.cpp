@@ -214,73 +214,113 @@ int64_t hybrid_top(const Tensor &signature, int64_t depth, int64_t d, bool alt, 
     return top;
 }
 
-std::tuple<Tensor, Tensor> sig_to_logsig_hip(const Tensor &signature_in, int64_t depth, int64_t d, bool alt,
-                                             const Tensor &encoded_words, at::IntArrayRef level_sizes) {
-    TORCH_CHECK(signature_in.is_cuda(), "signature must be CUDA");
-    const int dt = dtype_code(signature_in, "signature");
+// arguments shared by the log-signature operators: the hybrid-layout tensor `like` fixes rows and columns
+struct LogCall {
+    Tensor words;
+    int dt;
+    int64_t depth, d, top, S, rows;
+};
+
+LogCall log_call(const Tensor &like, const char *what, int64_t depth, int64_t d, bool alt, const Tensor &encoded_words,
+                 at::IntArrayRef level_sizes) {
+    LogCall c;
+    TORCH_CHECK(like.is_cuda(), what, " must be CUDA");
+    c.dt = dtype_code(like, what);
     TORCH_CHECK(depth >= 1 && depth <= PATHSIG_MAX_DEPTH, "depth must be in [1,12]");
     TORCH_CHECK(d >= 1, "d must be >= 1");
-    TORCH_CHECK(signature_in.dim() == 2 || signature_in.dim() == 3, "signature must be [B,S] or [B,W,S]");
-    Tensor sig = signature_in.contiguous();
-    Tensor words;
+    TORCH_CHECK(like.dim() == 2 || like.dim() == 3, what, " must be [B,S] or [B,W,S]");
+    c.depth = depth;
+    c.d = d;
     if (alt) {
         check_words_arg(encoded_words);
-        words = encoded_words.contiguous();
+        c.words = encoded_words.contiguous();
     }
-    const int64_t top = hybrid_top(sig, depth, d, alt, level_sizes);
-    if (words.defined() && top != dense_size(d, depth, depth)) {
-        TORCH_CHECK(words.numel() >= top, "encoded_words is shorter than the top level");
+    c.top = hybrid_top(like, depth, d, alt, level_sizes);
+    if (c.words.defined() && c.top != dense_size(d, depth, depth)) {
+        TORCH_CHECK(c.words.numel() >= c.top, "encoded_words is shorter than the top level");
     }
-    const int64_t S = sig.size(-1);
-    const int64_t rows = S > 0 ? sig.numel() / S : 0;
+    c.S = like.size(-1);
+    c.rows = c.S > 0 ? like.numel() / c.S : 0;
+    return c;
+}
+
+std::vector<int64_t> cache_shape_of(const Tensor &sig, int64_t depth) {
+    std::vector<int64_t> shape(sig.sizes().begin(), sig.sizes().end());
+    shape.back() = sig.size(-1) * depth;
+    return shape;
+}
+
+// keep: the second output is the cache the adjoint reads (powers of the log-signature) instead of the power
+// cache of the reference
+std::tuple<Tensor, Tensor> logsig_forward(const Tensor &signature_in, int64_t depth, int64_t d, bool alt,
+                                          const Tensor &encoded_words, at::IntArrayRef level_sizes, bool keep) {
+    const LogCall c = log_call(signature_in, "signature", depth, d, alt, encoded_words, level_sizes);
+    Tensor sig = signature_in.contiguous();
     c10::DeviceGuard guard(sig.device());
     Tensor logsig = at::empty_like(sig);
-    std::vector<int64_t> cache_shape(sig.sizes().begin(), sig.sizes().end());
-    cache_shape.back() = S * depth;
-    Tensor P = at::empty(cache_shape, sig.options());
-    check_rc(pathsig_logsig_forward(ptr(sig), ptr(logsig), ptr(P), dt, rows, d, (int)depth, top,
-                                    (const int64_t *)ptr(words), stream_of(sig)));
-    return {logsig, P};
+    Tensor cache = at::empty(cache_shape_of(sig, depth), sig.options());
+    if (keep)
+        check_rc(pathsig_logsig_forward_keep(ptr(sig), ptr(logsig), ptr(cache), c.dt, c.rows, d, (int)depth, c.top,
+                                             (const int64_t *)ptr(c.words), stream_of(sig)));
+    else
+        check_rc(pathsig_logsig_forward(ptr(sig), ptr(logsig), ptr(cache), c.dt, c.rows, d, (int)depth, c.top,
+                                        (const int64_t *)ptr(c.words), stream_of(sig)));
+    return {logsig, cache};
+}
+
+std::tuple<Tensor, Tensor> sig_to_logsig_hip(const Tensor &signature_in, int64_t depth, int64_t d, bool alt,
+                                             const Tensor &encoded_words, at::IntArrayRef level_sizes) {
+    return logsig_forward(signature_in, depth, d, alt, encoded_words, level_sizes, false);
+}
+
+std::tuple<Tensor, Tensor> sig_to_logsig_keep_hip(const Tensor &signature_in, int64_t depth, int64_t d, bool alt,
+                                                  const Tensor &encoded_words, at::IntArrayRef level_sizes) {
+    return logsig_forward(signature_in, depth, d, alt, encoded_words, level_sizes, true);
+}
+
+// first_in is the signature (kept == false; cache_in is then the reference's P, which is only checked for its
+// shape) or the log-signature of the keeping forward (kept == true; cache_in is its cache)
+Tensor logsig_backward_any(const Tensor &first_in, const Tensor &cache_in, const Tensor &grad_logsig_in, int64_t depth,
+                           bool alt, const Tensor &encoded_words, at::IntArrayRef level_sizes, bool kept) {
+    const char *first_name = kept ? "logsig" : "sig";
+    TORCH_CHECK(cache_in.is_cuda(), kept ? "cache" : "P", " must be CUDA");
+    TORCH_CHECK(grad_logsig_in.is_cuda(), "grad_logsig must be CUDA");
+    TORCH_CHECK((int64_t)level_sizes.size() > depth && depth >= 1, "level_sizes must have entries up to depth");
+    const int64_t d = level_sizes[1];  // the path dimension is read off the (always dense) first level
+    TORCH_CHECK(d >= 1, "level_sizes[1] must be >= 1 (infers path_dim)");
+    const LogCall c = log_call(first_in, first_name, depth, d, alt, encoded_words, level_sizes);
+    TORCH_CHECK(cache_in.scalar_type() == first_in.scalar_type(), "P must have same dtype as sig");
+    TORCH_CHECK(grad_logsig_in.scalar_type() == first_in.scalar_type(), "grad_logsig must have same dtype as sig");
+    Tensor first = first_in.contiguous();
+    Tensor cache = cache_in.contiguous();
+    Tensor grad = grad_logsig_in.contiguous();
+    TORCH_CHECK(first.sizes() == grad.sizes(), "grad_logsig must match sig shape");
+    TORCH_CHECK(cache.sizes() == at::IntArrayRef(cache_shape_of(first, depth)), "P must be [..., S*depth]");
+    c10::DeviceGuard guard(first.device());
+    Tensor out = at::empty_like(first);
+    if (kept) {
+        const size_t ws_bytes = pathsig_logsig_backward_kept_workspace(c.dt, c.rows, d, (int)depth, c.top);
+        Tensor ws = scratch(ws_bytes, first);
+        check_rc(pathsig_logsig_backward_kept(ptr(first), ptr(cache), ptr(grad), ptr(out), c.dt, c.rows, d, (int)depth,
+                                              c.top, (const int64_t *)ptr(c.words), ptr(ws), ws_bytes,
+                                              stream_of(first)));
+    } else {
+        const size_t ws_bytes = pathsig_logsig_backward_workspace(c.dt, c.rows, d, (int)depth, c.top);
+        Tensor ws = scratch(ws_bytes, first);
+        check_rc(pathsig_logsig_backward(ptr(first), ptr(cache), ptr(grad), ptr(out), c.dt, c.rows, d, (int)depth, c.top,
+                                         (const int64_t *)ptr(c.words), ptr(ws), ws_bytes, stream_of(first)));
+    }
+    return out;
 }
 
 Tensor logsig_backward_hip(const Tensor &signature_in, const Tensor &P_in, const Tensor &grad_logsig_in, int64_t depth,
                            bool alt, const Tensor &encoded_words, at::IntArrayRef level_sizes) {
-    TORCH_CHECK(signature_in.is_cuda(), "sig must be CUDA");
-    TORCH_CHECK(P_in.is_cuda(), "P must be CUDA");
-    TORCH_CHECK(grad_logsig_in.is_cuda(), "grad_logsig must be CUDA");
-    const int dt = dtype_code(signature_in, "sig");
-    TORCH_CHECK(P_in.scalar_type() == signature_in.scalar_type(), "P must have same dtype as sig");
-    TORCH_CHECK(grad_logsig_in.scalar_type() == signature_in.scalar_type(), "grad_logsig must have same dtype as sig");
-    TORCH_CHECK(depth >= 1 && depth <= PATHSIG_MAX_DEPTH, "depth must be in [1,12]");
-    TORCH_CHECK((int64_t)level_sizes.size() > depth, "level_sizes must have entries up to depth");
-    const int64_t d = level_sizes[1];  // the path dimension is read off the (always dense) first level
-    TORCH_CHECK(d >= 1, "level_sizes[1] must be >= 1 (infers path_dim)");
-    Tensor sig = signature_in.contiguous();
-    Tensor P = P_in.contiguous();
-    Tensor grad = grad_logsig_in.contiguous();
-    TORCH_CHECK(sig.dim() == 2 || sig.dim() == 3, "sig must be [B,S] or [B,W,S]");
-    TORCH_CHECK(sig.sizes() == grad.sizes(), "grad_logsig must match sig shape");
-    const int64_t S = sig.size(-1);
-    std::vector<int64_t> cache_shape(sig.sizes().begin(), sig.sizes().end());
-    cache_shape.back() = S * depth;
-    TORCH_CHECK(P.sizes() == at::IntArrayRef(cache_shape), "P must be [..., S*depth]");
-    Tensor words;
-    if (alt) {
-        check_words_arg(encoded_words);
-        words = encoded_words.contiguous();
-    }
-    const int64_t top = hybrid_top(sig, depth, d, alt, level_sizes);
-    if (words.defined() && top != dense_size(d, depth, depth)) {
-        TORCH_CHECK(words.numel() >= top, "encoded_words is shorter than the top level");
-    }
-    const int64_t rows = S > 0 ? sig.numel() / S : 0;
-    c10::DeviceGuard guard(sig.device());
-    Tensor out = at::empty_like(sig);
-    const size_t ws_bytes = pathsig_logsig_backward_workspace(dt, rows, d, (int)depth, top);
-    Tensor ws = scratch(ws_bytes, sig);
-    check_rc(pathsig_logsig_backward(ptr(sig), ptr(P), ptr(grad), ptr(out), dt, rows, d, (int)depth, top,
-                                     (const int64_t *)ptr(words), ptr(ws), ws_bytes, stream_of(sig)));
-    return out;
+    return logsig_backward_any(signature_in, P_in, grad_logsig_in, depth, alt, encoded_words, level_sizes, false);
+}
+
+Tensor logsig_backward_kept_hip(const Tensor &logsig_in, const Tensor &cache_in, const Tensor &grad_logsig_in,
+                                int64_t depth, bool alt, const Tensor &encoded_words, at::IntArrayRef level_sizes) {
+    return logsig_backward_any(logsig_in, cache_in, grad_logsig_in, depth, alt, encoded_words, level_sizes, true);
 }
 
 // ---- autograd (`src/pathsig/ops.py:231-297`) ---------------------------------------------------------------
@@ -382,6 +422,33 @@ struct LogSignatureFunction : public torch::autograd::Function<LogSignatureFunct
     }
 };
 
+// the same with the log-signature and its own cache handed to the backward (saves them instead of the signature)
+struct LogSignatureKeepFunction : public torch::autograd::Function<LogSignatureKeepFunction> {
+    static variable_list forward(AutogradContext *ctx, const Tensor &signature, int64_t depth, int64_t d, bool alt,
+                                 const Tensor &words, std::vector<int64_t> level_sizes) {
+        at::AutoDispatchBelowADInplaceOrView below;
+        static auto op = typed_op<LogForward>("pathsig::sig_to_logsig_keep");
+        auto [logsig, cache] = op.call(signature, depth, d, alt, words, level_sizes);
+        ctx->save_for_backward({logsig, cache, words});
+        ctx->saved_data["depth"] = depth;
+        ctx->saved_data["alt"] = alt;
+        ctx->saved_data["level_sizes"] = level_sizes;
+        ctx->set_materialize_grads(false);
+        ctx->mark_non_differentiable({cache});
+        return {logsig, cache};
+    }
+    static variable_list backward(AutogradContext *ctx, variable_list grads) {
+        const auto saved = ctx->get_saved_variables();
+        Tensor grad_sig;
+        if (ctx->needs_input_grad(0) && grads[0].defined()) {
+            static auto op = typed_op<LogBackward>("pathsig::logsig_backward_kept");
+            grad_sig = op.call(saved[0], saved[1], grads[0], ctx->saved_data["depth"].toInt(),
+                               ctx->saved_data["alt"].toBool(), saved[2], ctx->saved_data["level_sizes"].toIntVector());
+        }
+        return {grad_sig, Tensor(), Tensor(), Tensor(), Tensor(), Tensor()};
+    }
+};
+
 Tensor compute_signature_autograd(const Tensor &path, int64_t depth, bool alt, const Tensor &words,
                                   at::IntArrayRef level_sizes, bool use_windows, const Tensor &windows) {
     return SignatureFunction::apply(path, depth, alt, words, level_sizes.vec(), use_windows, windows);
@@ -397,6 +464,12 @@ std::tuple<Tensor, Tensor> compute_signature_keep_autograd(const Tensor &path, i
 std::tuple<Tensor, Tensor> sig_to_logsig_autograd(const Tensor &signature, int64_t depth, int64_t d, bool alt,
                                                   const Tensor &words, at::IntArrayRef level_sizes) {
     auto out = LogSignatureFunction::apply(signature, depth, d, alt, words, level_sizes.vec());
+    return {out[0], out[1]};
+}
+
+std::tuple<Tensor, Tensor> sig_to_logsig_keep_autograd(const Tensor &signature, int64_t depth, int64_t d, bool alt,
+                                                       const Tensor &words, at::IntArrayRef level_sizes) {
+    auto out = LogSignatureKeepFunction::apply(signature, depth, d, alt, words, level_sizes.vec());
     return {out[0], out[1]};
 }
 
@@ -420,6 +493,12 @@ TORCH_LIBRARY(pathsig, m) {
     m.def("signature_backward_kept(Tensor path_in, Tensor signature_in, Tensor grad_signature_in, Tensor chunks, "
           "int depth, bool alternative_projection, Tensor encoded_words, int[] level_sizes, bool use_windows, "
           "Tensor windows) -> Tensor", pt2);
+    // not in the reference: the second output is the cache of the adjoint (powers of the log-signature), and the
+    // backward takes the log-signature and that cache instead of the signature and the power cache
+    m.def("sig_to_logsig_keep(Tensor signature_in, int depth, int d, bool alternative_projection, "
+          "Tensor encoded_words, int[] level_sizes) -> (Tensor, Tensor)", pt2);
+    m.def("logsig_backward_kept(Tensor logsig_in, Tensor cache_in, Tensor grad_logsig_in, int depth, "
+          "bool alternative_projection, Tensor encoded_words, int[] level_sizes) -> Tensor", pt2);
 }
 
 TORCH_LIBRARY_IMPL(pathsig, CUDA, m) {
@@ -429,10 +508,13 @@ TORCH_LIBRARY_IMPL(pathsig, CUDA, m) {
     m.impl("logsig_backward", &logsig_backward_hip);
     m.impl("compute_signature_keep", &compute_signature_keep_hip);
     m.impl("signature_backward_kept", &signature_backward_kept_hip);
+    m.impl("sig_to_logsig_keep", &sig_to_logsig_keep_hip);
+    m.impl("logsig_backward_kept", &logsig_backward_kept_hip);
 }
 
 TORCH_LIBRARY_IMPL(pathsig, Autograd, m) {
     m.impl("compute_signature", &compute_signature_autograd);
     m.impl("sig_to_logsig", &sig_to_logsig_autograd);
     m.impl("compute_signature_keep", &compute_signature_keep_autograd);
+    m.impl("sig_to_logsig_keep", &sig_to_logsig_keep_autograd);
 }

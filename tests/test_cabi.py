@@ -28,10 +28,11 @@ def test_header_functions_are_exported(lib):
     assert {"pathsig_sig_forward", "pathsig_sig_backward", "pathsig_logsig_forward", "pathsig_logsig_backward",
             "pathsig_sig_forward_workspace", "pathsig_sig_backward_workspace", "pathsig_logsig_backward_workspace",
             "pathsig_sig_chunks_bytes", "pathsig_sig_forward_keep", "pathsig_sig_backward_kept",
+            "pathsig_logsig_forward_keep", "pathsig_logsig_backward_kept", "pathsig_logsig_backward_kept_workspace",
             "pathsig_last_error", "pathsig_abi_version"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
-    assert lib.pathsig_abi_version() == 2
+    assert lib.pathsig_abi_version() == 3
 
 
 def _fwd(lib, dtype=0, B=2, L=5, d=3, depth=3, path=1, sig=1, sizes=None):
@@ -56,12 +57,25 @@ def test_argument_errors_have_codes_and_messages(lib):
     rc = lib.pathsig_sig_backward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0,
                                   2, 5, 3, 3, None, None, 0, None, 0, None, 0, None)
     assert rc == ERR_WORKSPACE and b"workspace" in lib.pathsig_last_error()
+    # backward with a NULL signature or upstream gradient (a kernel would dereference them)
+    ws = ctypes.c_void_p(1)
+    for sig_ptr, grad_ptr in ((0, 1), (1, 0)):
+        rc = lib.pathsig_sig_backward(ctypes.c_void_p(1), ctypes.c_void_p(sig_ptr), ctypes.c_void_p(grad_ptr),
+                                      ctypes.c_void_p(1), 0, 2, 5, 3, 3, None, None, 0, None, 0, ws, 1 << 20, None)
+        assert rc == ERR_ARG and b"sig and grad_sig" in lib.pathsig_last_error()
     # log-signature entry points
     assert lib.pathsig_logsig_forward(None, None, None, 0, 4, 3, 3, 27, None, None) == ERR_ARG
     assert lib.pathsig_logsig_forward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0, 4, 3, 3, 5, None,
                                       None) == ERR_ARG  # listed top level without its codes
     assert lib.pathsig_logsig_forward(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1), 0, 4, 3, 0, 0, None,
                                       None) == ERR_ARG
+    assert lib.pathsig_logsig_forward_keep(ctypes.c_void_p(1), ctypes.c_void_p(1), None, 0, 4, 3, 3, 27, None,
+                                           None) == ERR_ARG and b"cache" in lib.pathsig_last_error()
+    assert lib.pathsig_logsig_backward_kept(ctypes.c_void_p(1), ctypes.c_void_p(1), ctypes.c_void_p(1),
+                                            ctypes.c_void_p(1), 0, 4, 3, 3, 27, None, None, 0, None) == ERR_WORKSPACE
+    # the plain adjoint rebuilds the log-signature and its cache in the workspace: it asks for more than the kept one
+    assert lib.pathsig_logsig_backward_workspace(0, 4, 3, 3, 27) >= \
+        lib.pathsig_logsig_backward_kept_workspace(0, 4, 3, 3, 27) + 4 * 39 * 4 * 4
     # empty batches are a no-op
     assert _fwd(lib, B=0, path=0, sig=0) == 0
     assert lib.pathsig_logsig_forward(None, None, None, 0, 0, 3, 3, 27, None, None) == 0

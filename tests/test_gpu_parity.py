@@ -294,6 +294,29 @@ def test_sig_to_logsig_cache_layout(ps):
     assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
 
 
+def test_sig_to_logsig_keep_cache(ps):
+    """The keeping forward returns the same log-signature and, as its cache, the tensor powers of that
+    log-signature (entry k - 1 of a word's row: its coefficient in L^(x)k); the kept backward agrees with the
+    checker's adjoint."""
+    d, depth, B = 3, 4, 2
+    top = [5, 80, 17, 17, 2]
+    path = brownian_path(B, 9, d, seed=45) * 1.5
+    dense = TO.signature(path, depth)
+    cols = TO.hybrid_columns(d, depth, len(top), top)
+    hyb = dense[:, cols]
+    want_log, _ = TO.sig_to_logsig(hyb, depth, d, len(top), top)
+    want_cache = TO.logsig_power_cache(want_log, depth, d, len(top), top)
+    sizes = [0] + [d ** k for k in range(1, depth)] + [len(top)]
+    words = torch.tensor(top, dtype=torch.int64, device=DEV)
+    logsig, cache = torch.ops.pathsig.sig_to_logsig_keep(hyb.to(DEV), depth, d, True, words, sizes)
+    assert cache.shape == (B, len(cols) * depth)
+    assert rel_err(logsig, want_log) < 1e-12
+    assert rel_err(cache, want_cache) < 1e-12
+    g = randn(tuple(hyb.shape), seed=46)
+    got = torch.ops.pathsig.logsig_backward_kept(logsig, cache, g.to(DEV), depth, True, words, sizes)
+    assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
+
+
 @pytest.mark.parametrize("form", ["gather", "scatter"])
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("d,depth,top", [
@@ -305,12 +328,9 @@ def test_sig_to_logsig_cache_layout(ps):
     (8, 5, "lyndon"),                  # the size of the benchmark configuration
     (9, 5, None),                      # odd alphabet, dense top level of 59049 words
 ])
-def test_logsig_adjoint_both_forms(ps, monkeypatch, form, dtype, d, depth, top):
+def test_logsig_adjoint_both_forms(ps, set_option, form, dtype, d, depth, top):
     """The adjoint op against the checker, in its gather form and (forced) in its scatter form."""
-    if form == "scatter":
-        monkeypatch.setenv("PATHSIG_LOGSIG_SCATTER", "1")
-    else:
-        monkeypatch.delenv("PATHSIG_LOGSIG_SCATTER", raising=False)
+    set_option("logsig_scatter", 1 if form == "scatter" else 0)
     B = 5
     if top == "lyndon":
         proj = ps.projections.lyndon(depth=depth, path_dim=d)
@@ -328,6 +348,40 @@ def test_logsig_adjoint_both_forms(ps, monkeypatch, form, dtype, d, depth, top):
     got = torch.ops.pathsig.logsig_backward(hyb.to(dtype).to(DEV), P, g.to(dtype).to(DEV), depth, alt, words, sizes)
     want = TO.logsig_vjp(hyb, g, depth, d, n_top, top)
     assert rel_err(got, want) < TOL[dtype]
+    # the pair that hands the log-signature and its cache over instead of rebuilding them
+    logsig_k, cache = torch.ops.pathsig.sig_to_logsig_keep(hyb.to(dtype).to(DEV), depth, d, alt, words, sizes)
+    assert torch.equal(logsig_k, logsig)
+    got_k = torch.ops.pathsig.logsig_backward_kept(logsig_k, cache, g.to(dtype).to(DEV), depth, alt, words, sizes)
+    assert rel_err(got_k, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,L,scale,kind", [
+    (2, 7, 3, 2.0, "lyndon"), (2, 8, 3, 2.0, "lyndon"), (2, 8, 65, 2.0, "dense"), (2, 8, 130, 2.0, "dense"),
+    (2, 8, 130, 2.0, "lyndon"), (3, 6, 2, 2.0, "dense"), (3, 6, 200, 2.0, "dense"), (3, 7, 40, 2.0, "lyndon"),
+    (3, 8, 100, 3.0, "lyndon"), (2, 10, 50, 2.0, "lyndon"), (2, 12, 30, 2.0, "lyndon"), (3, 9, 20, 1.0, "lyndon"),
+])
+def test_logsignature_deep_and_long(ps, dtype, d, depth, L, scale, kind):
+    """Regimes where the powers of S - 1 reach 1e5 .. 1e7 while the log-signature stays O(10): summing the
+    alternating series of the reference in fp32 is off by 1e-4 .. 1e-3 there (its literal fp32 restatement in
+    oracle/ref_words.c shows the same), the inverted exponential series holds the fp32 tolerance.  Depths follow
+    the sweep of the reference's `tests/test_logsig.py:138-146` (depth 2..12 at d = 3, fp32 at 1e-5 / 1e-4)."""
+    B = 2
+    proj = ps.projections.lyndon(depth=depth, path_dim=d) if kind == "lyndon" else None
+    path = brownian_path(B, L, d, seed=300 + depth) * scale
+    cols = None if proj is None else torch.tensor(TO.projection_columns(d, depth, proj.level_sizes, proj._codes))
+    xr = path.clone().requires_grad_(True)
+    # checker: the logarithm by inverting the exponential (the alternating series of the reference, summed in
+    # fp64, is itself off by 1e-11 in these regimes; tests/test_oracle_math.py pins both against extended precision)
+    full = TO.logsignature(xr, depth, method="inverse_exp")
+    ref = full if cols is None else full.index_select(-1, cols)
+    G = randn(tuple(ref.shape), seed=301)
+    (ref_grad,) = torch.autograd.grad(ref, xr, G)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    out = ps.LogSignature(depth=depth, projection=proj)(x)
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    assert rel_err(out, ref.detach()) < TOL[dtype]
+    assert rel_err(grad, ref_grad) < 10 * TOL[dtype]
 
 
 # ------------------------------------------------------------------------------------------------
@@ -543,10 +597,10 @@ def test_tiled_shapes_with_windows(ps, dtype, d, depth):
 @pytest.mark.parametrize("chunks", ["2", "5", "16"])
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("d,depth", TILED)
-def test_tiled_shapes_time_chunked(ps, monkeypatch, chunks, dtype, d, depth):
+def test_tiled_shapes_time_chunked(ps, set_option, chunks, dtype, d, depth):
     """Long paths are cut into time chunks whose signatures are multiplied back together (Chen);
-    PATHSIG_CHUNKS forces the chunk count so that small inputs exercise that path too."""
-    monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
+    The "chunks" option forces the chunk count so that small inputs exercise that path too."""
+    set_option("chunks", int(chunks))
     B, L = 2, 150
     path = brownian_path(B, L, d, seed=400 + d + depth)
     want = TO.signature(path, depth)
@@ -558,10 +612,10 @@ def test_tiled_shapes_time_chunked(ps, monkeypatch, chunks, dtype, d, depth):
 
 @pytest.mark.parametrize("L", [2, 3, 5, 67])
 @pytest.mark.parametrize("d,depth", TILED)
-def test_tiled_shapes_more_chunks_than_increments(ps, monkeypatch, d, depth, L):
+def test_tiled_shapes_more_chunks_than_increments(ps, set_option, d, depth, L):
     """Chunks without increments, one-increment chunks, and chunks longer than a tile of the reverse sweep:
     the backward writes the path gradient chunk by chunk and must leave no point untouched."""
-    monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+    set_option("chunks", 4)
     B = 3
     path = brownian_path(B, L, d, seed=450 + d + depth + L)
     want = TO.signature(path, depth)
@@ -577,8 +631,8 @@ def test_tiled_shapes_more_chunks_than_increments(ps, monkeypatch, d, depth, L):
 
 
 @pytest.mark.parametrize("d,depth", [(4, 6), (6, 5)])
-def test_tiled_shapes_time_chunked_windows(ps, monkeypatch, d, depth):
-    monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+def test_tiled_shapes_time_chunked_windows(ps, set_option, d, depth):
+    set_option("chunks", 4)
     B, L = 2, 100
     path = brownian_path(B, L, d, seed=500 + d)
     wins = [(0, 100), (0, 64), (32, 96), (64, 100), (10, 12), (50, 50), (3, 80), (97, 100)]  # some shorter than the chunk count
@@ -636,7 +690,7 @@ def test_logsignature_lyndon_through_dense_kernels(ps, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("kind", ["irregular", "lyndon"])
-def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dtype, kind):
+def test_projection_through_dense_kernels_with_letter_bounds(ps, set_option, dtype, kind):
     """d = 8, depth 5: the sweeps leave out the top-level words whose later letters fall below the
     smallest one used after the same first letter.  The word list has a different bound per first letter,
     one first letter without words, and unordered, repeated words; the run without bounds must agree."""
@@ -667,9 +721,9 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dt
         got, grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
         assert rel_err(got, want) < TOL[dtype]
         assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes, windows)) < TOL[dtype]
-        monkeypatch.setenv("PATHSIG_NO_LETTER_BOUNDS", "1")
+        set_option("letter_bounds", 0)
         plain, plain_grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)
-        monkeypatch.delenv("PATHSIG_NO_LETTER_BOUNDS")
+        set_option("letter_bounds", 1)
         assert rel_err(got, plain) < TOL[dtype] and rel_err(grad, plain_grad) < TOL[dtype]
 
 
@@ -679,7 +733,7 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, monkeypatch, dt
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("case", ["dense", "windows", "lyndon", "not_chunked", "per_word", "words_few_paths",
                                   "words_many_paths", "words_windows"])
-def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, case):
+def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case):
     """`compute_signature_keep` / `signature_backward_kept` (what the modules use when a gradient is wanted)
     against the reference's pair `compute_signature` / `signature_backward`: same signature, same dL/dpath.
     Kept are the time-chunk signatures of the register-tiled kernels, or, on the per-word kernels, the prefix
@@ -690,15 +744,15 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, cas
     depth, kw, chunked = 4, {}, True
     if case == "dense":
         d, B, L = 4, 5, 300
-        monkeypatch.setenv("PATHSIG_CHUNKS", "5")
+        set_option("chunks", 5)
     elif case == "windows":
         d, B, L = 4, 3, 200
         kw["windows"] = [(0, 200), (10, 150), (40, 42), (7, 7)]
-        monkeypatch.setenv("PATHSIG_CHUNKS", "4")
+        set_option("chunks", 4)
     elif case == "lyndon":
         d, depth, B, L = 8, 5, 2, 90
         kw["projection"] = ps.projections.lyndon(depth=depth, path_dim=d, full_levels=(1, 2, 3, 4))
-        monkeypatch.setenv("PATHSIG_CHUNKS", "3")
+        set_option("chunks", 3)
     elif case == "not_chunked":
         d, B, L, chunked = 4, 3000, 20, False
     elif case == "per_word":
@@ -746,11 +800,11 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, monkeypatch, dtype, cas
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("chunks", [None, "4"])
-def test_shape_with_two_prefix_lengths(ps, monkeypatch, dtype, chunks):
+def test_shape_with_two_prefix_lengths(ps, set_option, dtype, chunks):
     """(d, depth) = (8, 4) is compiled with lanes on prefixes of length 2 and of length 3; small batches take the
     longer prefix (the other tests of this shape), a batch that fills the GPU takes the shorter one."""
     if chunks:
-        monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
+        set_option("chunks", int(chunks))
     d, depth, B, L = 8, 4, 200, 100
     path = brownian_path(B, L, d, seed=501)
     for windows in (None, [(0, 100), (10, 90), (50, 52)]):

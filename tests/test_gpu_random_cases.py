@@ -1,6 +1,7 @@
 """Seeded random cases against the level-tensor checker: shapes with and without a register-tiled kernel,
 both dtypes, windows (degenerate ones included), every projection builder, forced time-chunk counts, through the
-modules (forward that keeps its chunk signatures) and through the reference's stateless pair of ops."""
+modules (forward that keeps its chunk signatures) and through the reference's stateless pair of ops; then the
+log-signature of the same case (dense, Lyndon and anisotropic projections, windows, both dtypes)."""
 from __future__ import annotations
 
 import itertools
@@ -54,21 +55,18 @@ def _random_case(rng, ps):
             proj = None
     scale = rng.choice([0.5, 1.0, 2.0])
     seeds = (rng.randint(0, 10 ** 6), rng.randint(0, 10 ** 6))
-    return d, depth, B, L, dtype, proj, windows, chunks, scale, seeds
+    return d, depth, B, L, dtype, proj, windows, chunks, scale, seeds, kind
 
 
 @pytest.mark.parametrize("seed", [11, 12, 13])
-def test_random_signature_cases(monkeypatch, seed):
+def test_random_signature_cases(set_option, seed):
     import pathsig_amd as ps
     rng = random.Random(seed)
     for case in range(40):
-        d, depth, B, L, dtype, proj, windows, chunks, scale, seeds = _random_case(rng, ps)
+        d, depth, B, L, dtype, proj, windows, chunks, scale, seeds, kind = _random_case(rng, ps)
         if d ** depth > 40000:
             continue
-        if chunks:
-            monkeypatch.setenv("PATHSIG_CHUNKS", chunks)
-        else:
-            monkeypatch.delenv("PATHSIG_CHUNKS", raising=False)
+        set_option("chunks", int(chunks) if chunks else 0)
         sizes, codes = (None, None) if proj is None else (proj.level_sizes, proj._codes)
         path = brownian_path(B, L, d, seed=seeds[0]) * scale
         want = TO.compute_signature(path, depth, sizes, codes, windows)
@@ -91,3 +89,22 @@ def test_random_signature_cases(monkeypatch, seed):
             sig = torch.ops.pathsig.compute_signature(x, *args)
             grad = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)
         assert rel_err(sig, want) < tol and rel_err(grad, want_grad) < tol, what
+        if kind not in ("dense", "lyndon", "aniso") or d ** depth > 5000:
+            continue
+        # log-signature of the same case; the checker takes the logarithm of the dense signature (by inverting
+        # the exponential: the alternating series in fp64 is not good to 1e-12 on the deep and long cases) and selects
+        cols = None if proj is None else torch.tensor(TO.projection_columns(d, depth, sizes, codes))
+        xr = path.clone().requires_grad_(True)
+        if windows:
+            full = torch.stack([TO.logsignature(xr[:, s:e], depth, method="inverse_exp") if e - s >= 2
+                                else torch.zeros(B, TO.dense_size(d, depth), dtype=torch.float64)
+                                for s, e in windows], dim=1)
+        else:
+            full = TO.logsignature(xr, depth, method="inverse_exp")
+        ref = full if cols is None else full.index_select(-1, cols)
+        Gl = randn(tuple(ref.shape), seed=seeds[1] + 1)
+        ref_grad = torch.autograd.grad(ref, xr, Gl)[0] if ref.requires_grad else torch.zeros_like(path)
+        xl = path.to(dtype).to(DEV).requires_grad_(True)
+        lout = ps.LogSignature(depth=depth, projection=proj, windows=win)(xl)
+        (lgrad,) = torch.autograd.grad(lout, xl, Gl.to(dtype).to(DEV))
+        assert rel_err(lout, ref.detach()) < tol and rel_err(lgrad, ref_grad) < 5 * tol, "log-signature, " + what

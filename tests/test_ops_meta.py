@@ -73,21 +73,12 @@ def test_chunk_buffer_size_follows_the_library():
     assert ops._chunks_numel(_meta(4096, 20, 4), 6, False, [], 0) == 0       # short paths, many rows: one chunk
 
 
-def test_both_registrations_define_the_same_ops():
-    """The C++ registration (when built) and the Python one expose the same schemas."""
-    code = ("import torch, pathsig_amd; from pathsig_amd import ops; "
-            "print(int(ops._NATIVE_OPS)); "
-            "print('\\n'.join(str(getattr(torch.ops.pathsig, n).default._schema) for n in "
-            "('compute_signature','signature_backward','sig_to_logsig','logsig_backward',"
-            "'compute_signature_keep','signature_backward_kept')))")
-    outs = []
-    for env_value in ("", "1"):
-        env = dict(os.environ, PATHSIG_PYTHON_OPS=env_value)
-        if not env_value:
-            env.pop("PATHSIG_PYTHON_OPS")
-        res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300,
-                             cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-        assert res.returncode == 0, res.stderr
-        outs.append(res.stdout.strip().split("\n"))
-    assert outs[1][0] == "0"                      # forced Python registration
-    assert outs[0][1:] == outs[1][1:]
+def test_missing_operator_library_is_an_error(tmp_path):
+    """There is one registration (C++): a package copy without libpathsig_torch.so refuses to import."""
+    import shutil
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pkg = tmp_path / "pathsig_amd"
+    shutil.copytree(os.path.join(root, "pathsig_amd"), pkg, ignore=shutil.ignore_patterns("csrc", "__pycache__", "libpathsig_torch.so"))
+    res = subprocess.run([sys.executable, "-c", "import pathsig_amd"], capture_output=True, text=True, timeout=300,
+                         cwd=str(tmp_path))
+    assert res.returncode != 0 and "libpathsig_torch.so" in res.stderr

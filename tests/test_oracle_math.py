@@ -184,6 +184,49 @@ def test_log_then_exp_is_identity():
         assert (a - b).abs().max() < 1e-13
 
 
+def test_inverse_exp_log_is_the_same_function():
+    """`tensor_log_levels_inverse_exp`: exp of it is S (independent exponential), it equals the alternating series
+    on a well-conditioned input, and on an ill-conditioned one (powers of S - 1 up to 1e6) it is the series
+    summed in extended precision that it agrees with, not the series summed in fp64."""
+    import numpy as np
+
+    d, depth = 3, 5
+    S = TO.split_levels(TO.signature(randn((2, 7, d), seed=10), depth), d, depth)
+    L = TO.tensor_log_levels_inverse_exp(S, depth)
+    for a, b in zip(S, tensor_exp_levels(L, depth)):
+        assert (a - b).abs().max() < 1e-13
+    for a, b in zip(L, TO.tensor_log_levels(S, depth)):
+        assert (a - b).abs().max() < 1e-13
+
+    d, depth = 2, 8
+    sig = TO.signature(brownian_path(2, 130, d, seed=5) * 2.0, depth)
+    S = TO.split_levels(sig, d, depth)
+    series = torch.cat(TO.tensor_log_levels(S, depth), dim=-1)
+    inverse = torch.cat(TO.tensor_log_levels_inverse_exp(S, depth), dim=-1)
+    # the alternating series in x87 extended precision (64-bit mantissa), level tensors as numpy arrays
+    ld = np.longdouble
+    if np.finfo(ld).eps > 1e-18:
+        pytest.skip("no extended precision on this platform")
+    Sn = [x.numpy().astype(ld) for x in S]
+    powers = [list(Sn)]
+    for m in range(2, depth + 1):
+        prev, cur = powers[-1], []
+        for n in range(1, depth + 1):
+            acc = np.zeros_like(Sn[n - 1])
+            for k in range(m - 1, n):
+                acc = acc + (prev[k - 1][:, :, None] * Sn[n - k - 1][:, None, :]).reshape(acc.shape[0], -1)
+            cur.append(acc)
+        powers.append(cur)
+    exact = np.concatenate([sum(ld((-1.0) ** (m + 1)) / ld(m) * powers[m - 1][n - 1] for m in range(1, n + 1))
+                            for n in range(1, depth + 1)], axis=1).astype(np.float64)
+    scale = max(1.0, float(np.abs(exact).max()))
+    assert max(float(np.abs(p).max()) for pw in powers for p in pw) > 1e5      # the input is ill conditioned
+    err_inverse = np.abs(inverse.numpy() - exact).max() / scale
+    err_series = np.abs(series.numpy() - exact).max() / scale
+    assert err_inverse < 1e-13
+    assert err_series > 10 * err_inverse and err_series > 5e-13                # the fp64 series is the one off
+
+
 def test_log_closed_forms_and_lie_property():
     d, depth = 3, 4
     path = randn((1, 6, d), seed=11)
