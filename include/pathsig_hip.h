@@ -74,6 +74,22 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Signature backward that allocates nothing.  No counterpart in the reference: it is for callers that cannot
+ * call hipMalloc or bring a workspace -- code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  Same arguments and results as pathsig_sig_backward, without `workspace`: the scratch is a fixed
+ * array of PATHSIG_STATIC_SCRATCH_BYTES that lives in the library's device image (every GPU the library runs on
+ * holds one until the process ends).  A call that needs more (pathsig_sig_backward_workspace tells) fails with
+ * PATHSIG_ERR_WORKSPACE and launches nothing.  All calls on one GPU share that array: calls that overlap on one
+ * GPU (two streams, two threads) race; serialise them or use the entry point with a workspace.  The first call on
+ * a device looks the array's address up (hipGetSymbolAddress); make that call outside a graph capture.
+ */
+#define PATHSIG_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+int pathsig_sig_backward_noalloc(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                                 int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                                 const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                                 void *stream);
+
+/*
  * The same pair with a hand-over from the forward to the backward of one call (no counterpart in the
  * reference, whose backward receives the path and the signature only and recomputes what it needs).
  * On long paths the register-tiled kernels cut every row into time chunks; the forward can write the

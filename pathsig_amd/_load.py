@@ -47,6 +47,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pathsig_sig_backward.restype = _INT
     lib.pathsig_sig_backward.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _I64, _INT, _PTR, _PTR, _I64,
                                          _PTR, _I64, _PTR, _SIZE, _PTR]
+    lib.pathsig_sig_backward_noalloc.restype = _INT
+    lib.pathsig_sig_backward_noalloc.argtypes = [_PTR, _PTR, _PTR, _PTR, _INT, _I64, _I64, _I64, _INT, _PTR, _PTR, _I64,
+                                                 _PTR, _I64, _PTR]
     lib.pathsig_sig_chunks_bytes.restype = _SIZE
     lib.pathsig_sig_chunks_bytes.argtypes = [_INT, _I64, _I64, _I64, _INT, _PTR, _I64]
     lib.pathsig_sig_forward_keep.restype = _INT

@@ -5,8 +5,16 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "dense.hpp"
+
+// Scratch of the entry point that allocates nothing (pathsig_sig_backward_noalloc).  Every GPU that loads the
+// library holds its own copy of this array, at its own address, until the process ends.  In host code the name
+// below is only a handle for hipGetSymbolAddress: the address that kernels and fills receive is the one that
+// call returns for the current device (static_scratch_of_current_device).
+static __device__ __align__(256) unsigned char scratch[PATHSIG_STATIC_SCRATCH_BYTES];
 
 namespace psig {
 
@@ -411,6 +419,52 @@ int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig
                          void *workspace, size_t workspace_bytes, void *stream) {
     return pathsig_sig_backward_kept(path, sig, grad_sig, grad_path, dtype, B, L, d, depth, level_sizes, encoded_words,
                                      n_encoded, windows, W, nullptr, 0, workspace, workspace_bytes, stream);
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return launch_failed(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) {
+        set_error("device index %d is beyond the %d devices the static scratch is tracked for", dev, kMaxDevices);
+        return PATHSIG_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return launch_failed(e, "hipGetSymbolAddress(scratch)");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return PATHSIG_OK;
+}
+}  // namespace
+
+int pathsig_sig_backward_noalloc(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
+                                 int64_t B, int64_t L, int64_t d, int depth, const int64_t *level_sizes,
+                                 const int64_t *encoded_words, int64_t n_encoded, const int32_t *windows, int64_t W,
+                                 void *stream) {
+    int rc = check_common(dtype, B, L, d, depth);
+    if (rc != PATHSIG_OK) return rc;
+    const size_t need = pathsig_sig_backward_workspace(dtype, B, L, d, depth, level_sizes, windows ? W : 0);
+    if (need > (size_t)PATHSIG_STATIC_SCRATCH_BYTES) {
+        set_error("this call needs %zu bytes of scratch; the static buffer of pathsig_sig_backward_noalloc holds %zu "
+                  "(use pathsig_sig_backward with a workspace of your own)", need, (size_t)PATHSIG_STATIC_SCRATCH_BYTES);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    void *ws = nullptr;
+    rc = static_scratch_of_current_device(&ws);
+    if (rc != PATHSIG_OK) return rc;
+    // the backward clears every part of its workspace that has to start from zero
+    return pathsig_sig_backward(path, sig, grad_sig, grad_path, dtype, B, L, d, depth, level_sizes, encoded_words,
+                                n_encoded, windows, W, ws, (size_t)PATHSIG_STATIC_SCRATCH_BYTES, stream);
 }
 
 int pathsig_sig_backward_kept(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,
