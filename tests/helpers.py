@@ -26,6 +26,27 @@ def rel_err(a, b):
     return float((a - b).abs().max() / max(1.0, float(b.abs().max())))
 
 
+def strict_rel_err(a, b):
+    """max|a-b| / max|b| (no floor of 1 in the denominator: small quantities are held to the same relative bound)."""
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    scale = float(b.abs().max())
+    return float((a - b).abs().max() / scale) if scale > 0 else float((a - b).abs().max())
+
+
+def level_rel_errs(got, want, level_sizes):
+    """Per level k: max|got_k - want_k| / max|want_k| over the columns of that level (the last axis holds the levels
+    one after the other with the given sizes).  The global metric divides by the largest coefficient of all, which
+    on Brownian inputs sits in level 1 or 2 and hides the high levels, whose coefficients are 1e-3 .. 1e-6."""
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    errs, off = [], 0
+    for size in level_sizes:
+        if size > 0:
+            errs.append(strict_rel_err(got[..., off:off + size], want[..., off:off + size]))
+        off += size
+    assert off == want.shape[-1]
+    return errs
+
+
 def all_words(d, n):
     return list(itertools.product(range(d), repeat=n))
 

@@ -813,3 +813,28 @@ def test_shape_with_two_prefix_lengths(ps, set_option, dtype, chunks):
         got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
         assert rel_err(got, want) < TOL[dtype]
         assert rel_err(grad, TO.signature_vjp(path, G, depth, windows=windows)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("d,depth", [(4, 6), (6, 5)])
+def test_many_long_rows_fp32_one_chunk(ps, d, depth):
+    """2048 rows of 4096 points in fp32: with that many rows the register-tiled kernels fill the GPU without
+    cutting the paths into time chunks, so the uncompensated forward accumulation and the reverse reconstruction
+    S_t = S_{t+1} (x) exp(-dx_t) both run over all 4095 increments in one piece.  Two of the paths against the
+    per-word C checker in fp64, level by level."""
+    from oracle import words_oracle as WO
+    from tests.helpers import level_rel_errs, strict_rel_err
+    B, L, sub = 2048, 4096, 2
+    head = brownian_path(sub, L, d, seed=77)
+    rest = brownian_path(8, L, d, seed=78).repeat(B // 8, 1, 1)[:B - sub]
+    x = torch.cat([head, rest]).float().to(DEV).requires_grad_(True)
+    out = ps.Signature(depth=depth)(x)
+    want = WO.sig_forward(head, depth)
+    G_head = randn(tuple(want.shape), seed=79)
+    G = torch.cat([G_head, randn((8, want.shape[1]), seed=80).repeat(B // 8, 1)[:B - sub]]).float().to(DEV)
+    (grad,) = torch.autograd.grad(out, x, G)
+    assert rel_err(out[:sub], want) < 1e-5
+    errs = level_rel_errs(out[:sub], want, [d ** k for k in range(1, depth + 1)])
+    assert max(errs) < 2e-5, errs
+    want_grad = WO.sig_backward(head, want, G_head, depth)
+    assert rel_err(grad[:sub], want_grad) < 1e-5
+    assert strict_rel_err(grad[:sub], want_grad) < 2e-5
