@@ -10,7 +10,7 @@ import torch
 
 from oracle import tensor_oracle as TO
 from oracle import words_oracle as WO
-from tests.helpers import rel_err
+from tests.helpers import level_rel_errs, rel_err
 
 GOLD = pathlib.Path(__file__).resolve().parent / "golden"
 
@@ -94,6 +94,14 @@ def test_kernels_reproduce_fixtures(dtype, tol):
     dev = "cuda"
     gtol = tol * (10 if dtype == torch.float32 else 1)
 
+    def levels_ok(out, want, sizes):
+        # every level relative to its own largest coefficient (twice the global bound)
+        errs = level_rel_errs(out, want, sizes)
+        assert max(errs) < 2 * tol, errs
+
+    def dense_sizes(f):
+        return [f["path"].shape[2] ** k for k in range(1, f["depth"] + 1)]
+
     def run(mod, f):
         x = f["path"].to(dtype).to(dev).requires_grad_("grad_out" in f)
         out = mod(x)
@@ -105,12 +113,15 @@ def test_kernels_reproduce_fixtures(dtype, tol):
     f = load("c1_small")
     out, _ = run(ps.Signature(depth=f["depth"]), f)
     assert rel_err(out, f["sig"]) < tol
+    levels_ok(out, f["sig"], dense_sizes(f))
     f = load("c2_small")
     out, grad = run(ps.Signature(depth=f["depth"]), f)
     assert rel_err(out, f["sig"]) < tol and rel_err(grad, f["grad_path"]) < gtol
+    levels_ok(out, f["sig"], dense_sizes(f))
     f = load("c3_small")
     out, grad = run(ps.Signature(depth=f["depth"], windows=f["windows"].to(dev)), f)
     assert rel_err(out, f["sig"]) < tol and rel_err(grad, f["grad_path"]) < gtol
+    levels_ok(out, f["sig"], dense_sizes(f))
     f = load("c4_small")
     flat, lens = f["words_flat"].tolist(), f["word_lengths"].tolist()
     words, pos = [], 0
@@ -120,6 +131,7 @@ def test_kernels_reproduce_fixtures(dtype, tol):
     proj = ps.projections.words(words, depth=f["depth"], path_dim=16, full_levels=(1, 2))
     out, grad = run(ps.Signature(depth=f["depth"], projection=proj), f)
     assert rel_err(out, f["sig"]) < tol and rel_err(grad, f["grad_path"]) < gtol
+    levels_ok(out, f["sig"], proj.level_sizes[1:])
     f = load("c5_small")
     proj = ps.projections.lyndon(depth=f["depth"], path_dim=4)
     out, grad = run(ps.LogSignature(depth=f["depth"], projection=proj), f)
