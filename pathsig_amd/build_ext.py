@@ -18,7 +18,13 @@ INCLUDE = PKG.parent / "include"
 LIB = PKG / "libpathsig_hip.so"
 TORCH_LIB = PKG / "libpathsig_torch.so"
 
-SOURCES = ["api.hip", "words_kernels.hip", "batch_kernels.hip", "logsig_kernels.hip", "dense_kernels.hip"]
+# (source, object, extra flags).  dense_kernels.hip is compiled once per group of register-tiled shapes and once
+# for the table of shapes and the dispatch, so the shapes build in parallel (the largest objects come first).
+DENSE_GROUPS = 4
+UNITS = ([("dense_kernels.hip", f"dense_kernels_g{g}.o", [f"-DPSIG_GROUP={g}"]) for g in range(DENSE_GROUPS)]
+         + [("batch_kernels.hip", "batch_kernels.o", []), ("words_kernels.hip", "words_kernels.o", []),
+            ("logsig_kernels.hip", "logsig_kernels.o", []), ("dense_kernels.hip", "dense_kernels.o", []),
+            ("api.hip", "api.o", [])])
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -34,9 +40,10 @@ HIPCC_FLAGS = [
 ]
 
 
-def _compile(src: str, verbose: bool) -> pathlib.Path:
-    obj = CSRC / (src.rsplit(".", 1)[0] + ".o")
-    cmd = ["hipcc", *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+def _compile(unit, verbose: bool) -> pathlib.Path:
+    src, obj_name, extra = unit
+    obj = CSRC / obj_name
+    cmd = ["hipcc", *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -50,9 +57,9 @@ def _compile(src: str, verbose: bool) -> pathlib.Path:
     return obj
 
 
-def build(verbose: bool = False, jobs: int = 4) -> pathlib.Path:
+def build(verbose: bool = False, jobs: int = 8) -> pathlib.Path:
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda s: _compile(s, verbose), SOURCES))
+        objs = list(pool.map(lambda u: _compile(u, verbose), UNITS))
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -37,6 +37,17 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
                                  const int64_t *top_codes, int64_t top_count, const T *kept, void *workspace,
                                  hipStream_t stream);
 
+// The compiled shapes are dealt to kDenseGroups translation units (shape index modulo kDenseGroups); these are the
+// launch sequences of one group.  `bounds`: device array of letter bounds, or nullptr.
+constexpr int kDenseGroups = 4;
+template <int GROUP, typename T>
+hipError_t launch_dense_forward_group(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
+                                      const int *bounds, T *keep, void *workspace, hipStream_t stream);
+template <int GROUP, typename T>
+hipError_t launch_dense_backward_group(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
+                                       bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
+                                       const int *bounds, const T *kept, void *workspace, hipStream_t stream);
+
 // measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
 // the begin and the end of that kernel on its stream; a no-op while the hook is off)
 void profile_enable(bool on);

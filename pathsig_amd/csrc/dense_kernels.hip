@@ -25,6 +25,14 @@
 
 #include "dense.hpp"
 
+// This file is compiled once per group of shapes (-DPSIG_GROUP=g, g = 0 .. kDenseGroups-1: the kernels of the
+// shapes whose index is g modulo kDenseGroups and their launch sequences) and once without a group (the table
+// of shapes, the choice of a shape for a call, and the dispatch to the groups), so that the shapes compile in
+// parallel.
+#ifndef PSIG_GROUP
+#define PSIG_GROUP -1
+#endif
+
 namespace psig {
 
 namespace {
@@ -1210,7 +1218,9 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 // lane) is taken.
 #define PSIG_VARIANTS(X) \
     X(0, 4, 6, 3, 5, 4) X(1, 8, 4, 2, 3, 2) X(2, 6, 5, 3, 3, 3) X(3, 4, 4, 2, 3, 2) X(4, 3, 5, 3, 4, 3) \
-    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3) X(7, 8, 4, 3, 3, 2)
+    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3) X(7, 8, 4, 3, 3, 2) X(8, 3, 6, 3, 5, 4) X(9, 4, 5, 3, 4, 3) \
+    X(10, 5, 4, 2, 3, 2) X(11, 5, 5, 3, 4, 3) X(12, 5, 6, 4, 4, 4) X(13, 6, 4, 2, 3, 2) X(14, 7, 4, 2, 3, 2) \
+    X(15, 7, 5, 3, 3, 3)
 
 struct VariantInfo {
     int d, depth, block;
@@ -1226,6 +1236,7 @@ constexpr VariantInfo variant_info() {
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
 
+#if PSIG_GROUP < 0
 // Computes the letter bounds of the top-level word list into the head of *workspace and moves *workspace
 // past them; returns nullptr (and launches nothing) when the call does not use bounds.
 const int *stage_letter_bounds(const DenseChoice &dc, const int64_t *top_codes, int64_t top_count, int d, int depth,
@@ -1239,6 +1250,8 @@ const int *stage_letter_bounds(const DenseChoice &dc, const int64_t *top_codes, 
     return bounds;
 }
 
+#endif
+
 #define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P>(),
 constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
 #undef PSIG_INFO
@@ -1246,6 +1259,7 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 size_t pad256(size_t n) { return (n + 255) / 256 * 256; }
 
+#if PSIG_GROUP < 0
 struct SweepProfile {
     bool enabled = false, valid = false;
     hipEvent_t start = nullptr, stop = nullptr;
@@ -1273,6 +1287,8 @@ int pick_chunks(int64_t rows, int block, int64_t L) {
     if (c < 1) c = 1;
     return (int)c;
 }
+
+#endif
 
 template <typename T, int D, int N, int P, int GW>
 constexpr bool group_fits() {
@@ -1362,7 +1378,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     }
     if (rows == 0) return hipSuccess;
     if (chunks <= 1) {
-        profile_mark(true, stream);
+        profile_bracket(true, stream);
         if (accumulate)
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, false>), dim3((unsigned)rows), dim3(G::kBlock),
                                0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr, grad_inc, shape,
@@ -1371,7 +1387,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, false>), dim3((unsigned)rows),
                                dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr,
                                grad_inc, shape, 1);
-        profile_mark(false, stream);
+        profile_bracket(false, stream);
         return hipGetLastError();
     }
     if constexpr (N < 2) {
@@ -1420,7 +1436,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        profile_mark(true, stream);
+        profile_bracket(true, stream);
         bool launched = false;
         if constexpr (kBoundsOk) {
             if (bounds) {
@@ -1446,13 +1462,14 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
                                    grad_inc, shape, chunks, grad_path);
         }
         if (!accumulate) *wrote_path = true;
-        profile_mark(false, stream);
+        profile_bracket(false, stream);
         return hipGetLastError();
     }
 }
 
 }  // namespace
 
+#if PSIG_GROUP < 0
 void profile_bracket(bool begin, hipStream_t stream) { profile_mark(begin, stream); }
 
 void profile_enable(bool on) {
@@ -1517,13 +1534,6 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
     return dc;
 }
 
-#define PSIG_CASE_FWD(I, D, N, P, PC, PS) \
-    case I: return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace, stream);
-#define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
-    case I:                                                                                                        \
-        return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc.bwd_chunks, \
-                                            bounds, kept, workspace, stream);
-
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
                                 const int64_t *top_codes, int64_t top_count, T *keep, void *workspace,
@@ -1532,9 +1542,11 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
     if (keep && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
-    switch (dc.variant) {
-        PSIG_VARIANTS(PSIG_CASE_FWD)
-        default: return hipErrorNotSupported;
+    switch (dc.variant % kDenseGroups) {
+        case 0: return launch_dense_forward_group<0, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
+        case 1: return launch_dense_forward_group<1, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
+        case 2: return launch_dense_forward_group<2, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
+        default: return launch_dense_forward_group<3, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
     }
 }
 
@@ -1547,9 +1559,15 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
     if (kept && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
-    switch (dc.variant) {
-        PSIG_VARIANTS(PSIG_CASE_BWD)
-        default: return hipErrorNotSupported;
+    switch (dc.variant % kDenseGroups) {
+#define PSIG_GROUP_CASE(GI)                                                                                          \
+    return launch_dense_backward_group<GI, T>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc, bounds, \
+                                              kept, workspace, stream)
+        case 0: PSIG_GROUP_CASE(0);
+        case 1: PSIG_GROUP_CASE(1);
+        case 2: PSIG_GROUP_CASE(2);
+        default: PSIG_GROUP_CASE(3);
+#undef PSIG_GROUP_CASE
     }
 }
 
@@ -1562,5 +1580,54 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE
+
+#else  // the kernels and launch sequences of one group of shapes
+
+static_assert(PSIG_GROUP < kDenseGroups, "group index out of range");
+
+#define PSIG_CASE_FWD(I, D, N, P, PC, PS)                                                                         \
+    case I:                                                                                                       \
+        if constexpr (I % kDenseGroups == PSIG_GROUP)                                                             \
+            return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace, stream); \
+        break;
+#define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
+    case I:                                                                                                        \
+        if constexpr (I % kDenseGroups == PSIG_GROUP)                                                              \
+            return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape,       \
+                                                dc.bwd_chunks, bounds, kept, workspace, stream);                   \
+        break;
+
+template <int GROUP, typename T>
+hipError_t launch_dense_forward_group(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
+                                      const int *bounds, T *keep, void *workspace, hipStream_t stream) {
+    switch (dc.variant) {
+        PSIG_VARIANTS(PSIG_CASE_FWD)
+        default: break;
+    }
+    return hipErrorNotSupported;
+}
+
+template <int GROUP, typename T>
+hipError_t launch_dense_backward_group(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
+                                       bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
+                                       const int *bounds, const T *kept, void *workspace, hipStream_t stream) {
+    switch (dc.variant) {
+        PSIG_VARIANTS(PSIG_CASE_BWD)
+        default: break;
+    }
+    return hipErrorNotSupported;
+}
+
+#define PSIG_INSTANTIATE(T)                                                                                          \
+    template hipError_t launch_dense_forward_group<PSIG_GROUP, T>(const T *, T *, const SigShape &, const DenseChoice &, \
+                                                                  const int *, T *, void *, hipStream_t);            \
+    template hipError_t launch_dense_backward_group<PSIG_GROUP, T>(const T *, const T *, const T *, T *, T *, bool *,  \
+                                                                   const SigShape &, const DenseChoice &, const int *, \
+                                                                   const T *, void *, hipStream_t);
+PSIG_INSTANTIATE(float)
+PSIG_INSTANTIATE(double)
+#undef PSIG_INSTANTIATE
+
+#endif  // PSIG_GROUP
 
 }  // namespace psig

@@ -565,7 +565,7 @@ def test_gradcheck(ps):
 # ------------------------------------------------------------------------------------------------
 # shapes served by the register-tiled dense kernels (forward, backward, windows, long paths)
 # ------------------------------------------------------------------------------------------------
-TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8)]
+TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -756,7 +756,7 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
     elif case == "not_chunked":
         d, B, L, chunked = 4, 3000, 20, False
     elif case == "per_word":
-        d, B, L, chunked = 5, 3, 40, False          # no register-tiled shape for d = 5: per-word kernels, all dense
+        d, B, L, chunked = 9, 3, 40, False          # no register-tiled shape for d = 9: per-word kernels, all dense
     else:
         d, depth, L = 5, 5, 60
         B = 3 if case == "words_few_paths" else 20
@@ -780,13 +780,16 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
         0 if dtype == torch.float32 else 1, B, L, d, depth, sizes, 0 if wins is None else len(wins))
     grad_k = torch.ops.pathsig.signature_backward_kept(x, sig_k, G, chunks, *args)
     assert torch.equal(sig_k, sig)
-    assert rel_err(grad_k, grad) < TOL[dtype] * 0.1
+    # two runs of the per-word backward differ by the order of their float atomics (a few 1e-6 of the largest
+    # gradient in fp32 at 6561 words); the register-tiled backward is deterministic without windows
+    close = TOL[dtype] * (0.5 if case == "per_word" else 0.1)
+    assert rel_err(grad_k, grad) < close
     # the module takes the keeping pair when a gradient is wanted
     xg = x.clone().requires_grad_(True)
     out = mod(xg)
     assert out.grad_fn is not None and "keep" in out.grad_fn.name().lower()
     (grad_m,) = torch.autograd.grad(out, xg, G)
-    assert torch.equal(out.detach(), sig) and rel_err(grad_m, grad) < TOL[dtype] * 0.1
+    assert torch.equal(out.detach(), sig) and rel_err(grad_m, grad) < close
     # a chunk buffer of the wrong size is refused
     if chunked:
         with pytest.raises(RuntimeError, match="chunk buffer"):
