@@ -1220,7 +1220,10 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(0, 4, 6, 3, 5, 4) X(1, 8, 4, 2, 3, 2) X(2, 6, 5, 3, 3, 3) X(3, 4, 4, 2, 3, 2) X(4, 3, 5, 3, 4, 3) \
     X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3) X(7, 8, 4, 3, 3, 2) X(8, 3, 6, 3, 5, 4) X(9, 4, 5, 3, 4, 3) \
     X(10, 5, 4, 2, 3, 2) X(11, 5, 5, 3, 4, 3) X(12, 5, 6, 4, 4, 4) X(13, 6, 4, 2, 3, 2) X(14, 7, 4, 2, 3, 2) \
-    X(15, 7, 5, 3, 3, 3)
+    X(15, 7, 5, 3, 3, 3) X(16, 2, 2, 1, 1, 1) X(17, 3, 2, 1, 1, 1) X(18, 4, 2, 1, 1, 1) X(19, 5, 2, 1, 1, 1) \
+    X(20, 6, 2, 1, 1, 1) X(21, 7, 2, 1, 1, 1) X(22, 8, 2, 1, 1, 1) X(23, 2, 3, 2, 2, 1) X(24, 3, 3, 2, 2, 1) \
+    X(25, 4, 3, 2, 2, 1) X(26, 5, 3, 2, 2, 1) X(27, 6, 3, 2, 2, 1) X(28, 7, 3, 2, 2, 1) X(29, 8, 3, 2, 2, 1) \
+    X(30, 2, 4, 3, 3, 2) X(31, 3, 4, 3, 3, 2) X(32, 2, 5, 4, 4, 3) X(33, 2, 6, 4, 5, 4)
 
 struct VariantInfo {
     int d, depth, block;
@@ -1390,7 +1393,8 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         profile_bracket(false, stream);
         return hipGetLastError();
     }
-    if constexpr (N < 2) {
+    if constexpr (N < 3) {
+        // depth 1 and 2 are never cut into time chunks (dense_choice): a row costs a few instructions per increment
         return hipErrorNotSupported;
     } else {
         const int64_t units = rows * chunks;
@@ -1506,7 +1510,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         if (!all_dense) {
             // A word projection is worth computing densely when its top level keeps a fair share of the
             // words (the top level dominates the cost) and the dense rows fit comfortably in memory.
-            if (!level_sizes) return dc;
+            if (!level_sizes || depth < 3) return dc;  // an embedded projection needs the time-chunked backward
             const int64_t top_dense = v.sig_size - v.low_size;
             if (level_sizes[depth] * 8 < top_dense) return dc;
             if ((double)rows * (double)v.sig_size * (double)elem > 4e9) return dc;
@@ -1517,6 +1521,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         }
         int chunks = pick_chunks(rows, v.block, L);
         if (const int64_t forced = options().chunks; forced >= 1 && forced <= 1024) chunks = (int)forced;
+        if (depth < 3) chunks = 1;  // the chunked backward needs a level below the top to scan over
         if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
         dc.variant = i;

@@ -565,7 +565,8 @@ def test_gradcheck(ps):
 # ------------------------------------------------------------------------------------------------
 # shapes served by the register-tiled dense kernels (forward, backward, windows, long paths)
 # ------------------------------------------------------------------------------------------------
-TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5)]
+TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5),
+         (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])

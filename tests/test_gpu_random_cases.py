@@ -16,7 +16,7 @@ from tests.helpers import brownian_path, randn, random_word_set, rel_err
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (8, 5), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5)]
-OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6), (6, 3)]
+OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6), (6, 3), (9, 4), (12, 2)]
 
 
 def _random_case(rng, ps):
