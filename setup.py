@@ -3,8 +3,13 @@ Python package around them.
 
 Counterpart of the reference's CMake build (`CMakeLists.txt`, `pyproject.toml`): `pip install .` or
 `python setup.py build_py` compiles the HIP sources in-tree first; nothing is fetched.
+
+The distribution installs the package under the reference's import name, `pathsig` (the source directory is
+`pathsig_amd/`), so `import pathsig` and `from pathsig import Signature, LogSignature, projections` work
+unchanged.  `PATHSIG_SKIP_NATIVE_BUILD=1` reuses the libraries already built in-tree instead of compiling.
 """
 import importlib.util
+import os
 import pathlib
 
 from setuptools import setup
@@ -23,7 +28,11 @@ def _build_library():
 
 class BuildWithHip(build_py):
     def run(self):
-        _build_library()
+        if not os.environ.get("PATHSIG_SKIP_NATIVE_BUILD"):
+            _build_library()
+        for lib in ("libpathsig_hip.so", "libpathsig_torch.so"):
+            if not (ROOT / "pathsig_amd" / lib).is_file():
+                raise RuntimeError(f"pathsig_amd/{lib} is not built")
         super().run()
 
 
@@ -31,8 +40,9 @@ setup(
     name="pathsig-amd",
     version="0.1.0",
     description="Path signature and log-signature operators for AMD MI355X (gfx950), drop-in for pathsig",
-    packages=["pathsig_amd"],
-    package_data={"pathsig_amd": ["libpathsig_hip.so", "libpathsig_torch.so", "csrc/*.hip", "csrc/*.hpp", "csrc/*.cpp"]},
+    packages=["pathsig"],
+    package_dir={"pathsig": "pathsig_amd"},
+    package_data={"pathsig": ["libpathsig_hip.so", "libpathsig_torch.so", "csrc/*.hip", "csrc/*.hpp", "csrc/*.cpp"]},
     data_files=[("include", ["include/pathsig_hip.h"])],
     python_requires=">=3.10",
     install_requires=["torch>=2.4"],
