@@ -25,9 +25,12 @@ constexpr int kBatchBlock = kBatchWaves * kWave;
 constexpr int kBatchStride = kWave + 1;
 constexpr int kBatchChunks = 2;  // a tile holds at most kBatchChunks * 64 increments x letters per path
 
-// words swept at once by one lane: chosen so that a wave has about the same work at every word length
+// words swept at once by one lane: chosen so that a wave has about the same work at every word length.  Every
+// block pays the same fixed cost per increment (staging, slab flush, barriers), whatever its words cost, and the
+// slabs allow one block per CU: the short words of levels 1 and 2 are therefore packed sixteen to a lane, which
+// keeps a projection like "two full levels + a few thousand words" within one round of blocks on 256 CUs.
 constexpr int batch_words(int deg) {
-    return deg <= 3 ? 8 : deg == 4 ? 6 : deg == 5 ? 4 : deg == 6 ? 3 : deg <= 8 ? 2 : 1;
+    return deg <= 2 ? 16 : deg == 3 ? 8 : deg == 4 ? 6 : deg == 5 ? 4 : deg == 6 ? 3 : deg <= 8 ? 2 : 1;
 }
 
 // level of block `blk` when the levels are laid out from the deepest down: level k owns
