@@ -300,7 +300,8 @@ __device__ __forceinline__ T row_totals(T (&v)[D], int lane) {
 template <int D, int P>
 struct LetterBounds {
     static constexpr int kPerLetter = ipow(D, P - 1);  // lanes that share a first letter
-    static constexpr bool kUsable = P >= 1 && kPerLetter % kWave == 0;
+    // (units of more than 1024 lanes take several blocks and are swept without bounds)
+    static constexpr bool kUsable = P >= 1 && kPerLetter % kWave == 0 && ipow(D, P) <= 1024;
     static __device__ __forceinline__ int of_wave(const int *__restrict__ bounds, int pu) {
         const int first = __builtin_amdgcn_readfirstlane(pu / kPerLetter);
         const int lo = bounds[first];
@@ -396,8 +397,13 @@ constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2
 template <int D, int N, int P>
 struct Geometry {
     static constexpr int kLanes = ipow(D, P);
-    static constexpr int kWaves = (kLanes + kWave - 1) / kWave;
+    // A unit needs kUnitWaves waves.  Up to sixteen of them form one block; a larger unit is spread over
+    // kUnitBlocks blocks (its lanes never talk to each other inside a sweep; the per-increment sums of the
+    // backward then meet in memory).  Such shapes are swept in one piece, without time chunks.
+    static constexpr int kUnitWaves = (kLanes + kWave - 1) / kWave;
+    static constexpr int kWaves = kUnitWaves < 16 ? kUnitWaves : 16;  // waves of one block
     static constexpr int kBlock = kWaves * kWave;
+    static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
     static constexpr int kFwdSub = trie_size(D, N - P);    // sub-trie levels P+1..N
     static constexpr int kASub = trie_size(D, N - 1 - P);  // levels P+1..N-1
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
@@ -603,7 +609,8 @@ template <typename T, int D, int N, int P, int GW, int BOUND>
 __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T *__restrict__ out,
                                                    const SigShape &shape, int chunks, T *__restrict__ zero_rows,
                                                    T *__restrict__ chunk_low,
-                                                   const int pu,  // prefix of the thread within its chunk
+                                                   const int pu,   // prefix of the thread within its chunk
+                                                   const int tid,  // index of the thread within its chunk's block part
                                                    T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW>::kStage],
                                                    T (&slot)[ForwardShape<T, D, N, P, GW>::kSlots]
                                                             [ForwardShape<T, D, N, P, GW>::kSlotSize]) {
@@ -616,7 +623,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
     prefix_letters<D, P>(active ? pu : 0, u);
 
     const int groups = chunks / GW;  // blocks per row
-    const int64_t blk = blockIdx.x;
+    const int64_t blk = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
     const int64_t row = blk / groups;
     const int c = (int)(blk - row * groups) * GW + part;
     const int64_t b = row / shape.W, w = row - b * shape.W;
@@ -631,7 +638,8 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
         if (zero_rows) {
             const int64_t points = end - begin + (c == chunks - 1 ? 1 : 0);
             T *z = zero_rows + (b * shape.L + span.start + begin) * D;
-            for (int64_t idx = pu; idx < points * D; idx += G::kBlock) z[idx] = T(0);
+            if (pu == tid)  // the first block of the unit
+                for (int64_t idx = tid; idx < points * D; idx += G::kBlock) z[idx] = T(0);
         }
     }
 
@@ -648,7 +656,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
         const int nt = (int)(left < 0 ? 0 : (left < kTile ? left : kTile));
         const T *xw = x + t0 * D;
         lds_barrier();
-        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, pu);
+        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, tid);
         lds_barrier();
         if (nt > 0) {
             // two register sets of increments: the LDS reads of the next step are issued before the
@@ -700,16 +708,19 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
     __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
-    const int tid = (int)threadIdx.x % Geometry<D, N, P>::kBlock;
+    using G = Geometry<D, N, P>;
+    static_assert(G::kUnitBlocks == 1 || (GW == 1 && !BOUNDED), "a unit of several blocks is swept one chunk to a block");
+    const int tid = (int)threadIdx.x % G::kBlock;
     if constexpr (BOUNDED) {
         const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_forward_body<T, D, N, P, GW, decltype(loc)::value>(path, out, shape, chunks, zero_rows, chunk_low, pu,
-                                                                     sdx_all, slot);
+                                                                     tid, sdx_all, slot);
         });
     } else {
-        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, chunk_low, tid, sdx_all, slot);
+        const int pu = G::kUnitBlocks > 1 ? tid + (int)(blockIdx.x % G::kUnitBlocks) * G::kBlock : tid;
+        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, chunk_low, pu, tid, sdx_all, slot);
     }
 }
 
@@ -992,7 +1003,8 @@ template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, int BO
 __device__ __forceinline__ void dense_backward_body(
     const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig, const T *__restrict__ edgeA,
     const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
-    const int pu,  // prefix of the thread
+    const int pu,   // prefix of the thread
+    const int tid,  // index of the thread within its block
     T (&sdx)[BackwardShape<T, D, N, P>::kStage],
     T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
     T (&cells)[BackwardShape<T, D, N, P>::kCells]) {
@@ -1002,20 +1014,20 @@ __device__ __forceinline__ void dense_backward_body(
     constexpr int kParts = BS::kParts;
     constexpr int kBwdTile = BS::kBwdTile;
     constexpr bool kToPath = CHUNKED && !ACCUMULATE;  // writes the path gradient itself (see the tile flush)
-    const int lane = pu & (kWave - 1);
-    const int wave = pu / kWave;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;  // within the block
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
     // chain terms through LDS (see BackwardShape): the lane's cells start at zero
     constexpr bool kCellChain = BS::kChainCells && !(sizeof(T) == 4 && P * D <= 24);
-    T *my_cells = cells + (BS::kChainCells ? (int)threadIdx.x : 0);  // cell of letter k: my_cells[k * G::kBlock]
+    T *my_cells = cells + (BS::kChainCells ? tid : 0);  // cell of letter k: my_cells[k * G::kBlock]
     if constexpr (kCellChain) {
 #pragma unroll
         for (int k = 0; k < D; ++k) my_cells[k * G::kBlock] = T(0);
     }
 
-    const int64_t unit = blockIdx.x;
+    const int64_t unit = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
     const int64_t row = unit / chunks;
     const int c = (int)(unit - row * chunks);
     const int64_t b = row / shape.W, w = row - b * shape.W;
@@ -1061,7 +1073,7 @@ __device__ __forceinline__ void dense_backward_body(
         const int nt = (int)((end - t0) < kBwdTile ? (end - t0) : kBwdTile);
         const T *xw = x + t0 * D;
         lds_barrier();
-        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, (int)threadIdx.x);
+        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, tid);
         lds_barrier();
         auto step = [&](int tt, const T (&dxs)[KS][D], const T (&dxp)[P]) {
             // A_t = A_{t+1} (x) exp(-dx_t), levels < N
@@ -1150,7 +1162,7 @@ __device__ __forceinline__ void dense_backward_body(
             // Differences inside the tile are stored; the two ends of the tile are added to cells that the
             // chunk-signature launch has cleared and that receive exactly one more term from the
             // neighbouring tile (or none at the ends of the path), so the result does not depend on the order.
-            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+            for (int idx = tid; idx < nt * D; idx += G::kBlock) {
                 T v = sg[0][idx];
 #pragma unroll
                 for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
@@ -1158,14 +1170,14 @@ __device__ __forceinline__ void dense_backward_body(
             }
             lds_barrier();
             T *gp = grad_path + (b * shape.L + span.start + t0) * D;
-            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+            for (int idx = tid; idx < nt * D; idx += G::kBlock) {
                 const T cur = sg[0][idx];
                 if (idx >= D) gp[idx] = sg[0][idx - D] - cur;
                 else atomicAdd(&gp[idx], -cur);
                 if (idx >= (nt - 1) * D) atomicAdd(&gp[idx + D], cur);
             }
         } else {
-            for (int idx = threadIdx.x; idx < nt * D; idx += G::kBlock) {
+            for (int idx = tid; idx < nt * D; idx += G::kBlock) {
                 T v = sg[0][idx];
 #pragma unroll
                 for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
@@ -1193,16 +1205,21 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     __shared__ __align__(16) T sdx[BS::kStage];
     __shared__ T sg[BS::kSums][BS::kSumRow];
     __shared__ T cells[BS::kCells];
+    using G = Geometry<D, N, P>;
+    static_assert(G::kUnitBlocks == 1 || (ACCUMULATE && !CHUNKED && !BOUNDED),
+                  "a unit of several blocks is swept in one piece and adds its per-increment sums in memory");
+    const int tid = (int)threadIdx.x;
     if constexpr (BOUNDED) {
-        const int pu = LetterBounds<D, P>::prefix_of_thread((int)threadIdx.x);
+        const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value>(
-                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, sdx, sg, cells);
+                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells);
         });
     } else {
+        const int pu = G::kUnitBlocks > 1 ? tid + (int)(blockIdx.x % G::kUnitBlocks) * G::kBlock : tid;
         dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0>(path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape,
-                                                                chunks, grad_path, (int)threadIdx.x, sdx, sg, cells);
+                                                                chunks, grad_path, pu, tid, sdx, sg, cells);
     }
 }
 
@@ -1223,10 +1240,12 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(15, 7, 5, 3, 3, 3) X(16, 2, 2, 1, 1, 1) X(17, 3, 2, 1, 1, 1) X(18, 4, 2, 1, 1, 1) X(19, 5, 2, 1, 1, 1) \
     X(20, 6, 2, 1, 1, 1) X(21, 7, 2, 1, 1, 1) X(22, 8, 2, 1, 1, 1) X(23, 2, 3, 2, 2, 1) X(24, 3, 3, 2, 2, 1) \
     X(25, 4, 3, 2, 2, 1) X(26, 5, 3, 2, 2, 1) X(27, 6, 3, 2, 2, 1) X(28, 7, 3, 2, 2, 1) X(29, 8, 3, 2, 2, 1) \
-    X(30, 2, 4, 3, 3, 2) X(31, 3, 4, 3, 3, 2) X(32, 2, 5, 4, 4, 3) X(33, 2, 6, 4, 5, 4)
+    X(30, 2, 4, 3, 3, 2) X(31, 3, 4, 3, 3, 2) X(32, 2, 5, 4, 4, 3) X(33, 2, 6, 4, 5, 4) X(34, 6, 6, 4, 4, 3) \
+    X(35, 7, 6, 4, 4, 3) X(36, 8, 6, 4, 4, 3)
 
 struct VariantInfo {
-    int d, depth, block;
+    int d, depth, block;  // block: threads of one unit
+    int unit_blocks;      // blocks a unit is spread over (more than one: swept in one piece, dense only)
     int64_t sig_size, low_size;
     bool bounds_ok;  // the sweeps can leave out top-level words by letter bounds
 };
@@ -1234,7 +1253,8 @@ struct VariantInfo {
 template <int D, int N, int P>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
-    return VariantInfo{D, N, G::kBlock, G::kSigSize, G::kLowSize, LetterBounds<D, P>::kUsable && D <= 16};
+    return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
+                       LetterBounds<D, P>::kUsable && D <= 16};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1315,10 +1335,13 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                 return hipGetLastError();
             }
         }
-        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)rows), dim3(G::kBlock), 0, stream,
-                           path, sig, shape, 1);
+        hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)(rows * G::kUnitBlocks)),
+                           dim3(G::kBlock), 0, stream, path, sig, shape, 1);
         return hipGetLastError();
     }
+    if constexpr (G::kUnitBlocks > 1) {
+        return hipErrorNotSupported;  // such shapes are never cut into time chunks (dense_choice)
+    } else {
     // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits;
     // a row that fits one block goes straight to the output, without the combine launch
     T *chunk_sig = (T *)workspace;
@@ -1357,9 +1380,10 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
         hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, true>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
                            (const T *)chunk_sig, sig, groups);
     else
-        hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, false>), dim3((unsigned)rows, (unsigned)GC::kWaves),
+        hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, false>), dim3((unsigned)rows, (unsigned)GC::kUnitWaves),
                            dim3(kWave), 0, stream, (const T *)chunk_sig, sig, groups);
     return hipGetLastError();
+    }
 }
 
 template <typename T, int D, int N, int P, int PS>
@@ -1370,7 +1394,8 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     using GC = Geometry<D, N, PS>;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
     const int64_t rows = shape.B * shape.W;
-    const bool accumulate = shape.windows != nullptr;
+    // per-increment sums are added in memory for overlapping windows and for units spread over several blocks
+    const bool accumulate = shape.windows != nullptr || G::kUnitBlocks > 1;
     *wrote_path = false;
     hipError_t e;
     // bounded sweeps exist for time-chunked calls only (every call that embeds a projection is chunked)
@@ -1382,19 +1407,22 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     if (rows == 0) return hipSuccess;
     if (chunks <= 1) {
         profile_bracket(true, stream);
-        if (accumulate)
-            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, false>), dim3((unsigned)rows), dim3(G::kBlock),
-                               0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr, grad_inc, shape,
-                               1);
-        else
-            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, false>), dim3((unsigned)rows),
-                               dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)nullptr, (const T *)nullptr,
-                               grad_inc, shape, 1);
+        if (accumulate) {
+            hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, false>),
+                               dim3((unsigned)(rows * G::kUnitBlocks)), dim3(G::kBlock), 0, stream, path, sig, grad_sig,
+                               (const T *)nullptr, (const T *)nullptr, grad_inc, shape, 1);
+        } else {
+            if constexpr (G::kUnitBlocks == 1)
+                hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, false>), dim3((unsigned)rows),
+                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)nullptr,
+                                   (const T *)nullptr, grad_inc, shape, 1);
+        }
         profile_bracket(false, stream);
         return hipGetLastError();
     }
-    if constexpr (N < 3) {
-        // depth 1 and 2 are never cut into time chunks (dense_choice): a row costs a few instructions per increment
+    if constexpr (N < 3 || G::kUnitBlocks > 1) {
+        // depth 1 and 2 are never cut into time chunks (dense_choice): a row costs a few instructions per increment;
+        // nor are the shapes whose units take several blocks
         return hipErrorNotSupported;
     } else {
         const int64_t units = rows * chunks;
@@ -1507,6 +1535,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
         }
+        if (v.unit_blocks > 1 && !all_dense) return dc;
         if (!all_dense) {
             // A word projection is worth computing densely when its top level keeps a fair share of the
             // words (the top level dominates the cost) and the dense rows fit comfortably in memory.
@@ -1522,6 +1551,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         int chunks = pick_chunks(rows, v.block, L);
         if (const int64_t forced = options().chunks; forced >= 1 && forced <= 1024) chunks = (int)forced;
         if (depth < 3) chunks = 1;  // the chunked backward needs a level below the top to scan over
+        if (v.unit_blocks > 1) chunks = 1;  // a row of such a shape is dozens of waves already
         if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
         dc.variant = i;

@@ -842,3 +842,19 @@ def test_many_long_rows_fp32_one_chunk(ps, d, depth):
     want_grad = WO.sig_backward(head, want, G_head, depth)
     assert rel_err(grad[:sub], want_grad) < 1e-5
     assert strict_rel_err(grad[:sub], want_grad) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6)])
+def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
+    """d^6 for d >= 6: a row's lanes (d^4 prefixes) do not fit one block; the unit is spread over two to four
+    blocks, swept in one piece, and the per-increment sums of the backward meet in memory.  With and without
+    windows (overlapping ones included)."""
+    B, L = 2, 8
+    path = brownian_path(B, L, d, seed=500 + d) * 2.0
+    for windows in (None, [(0, 8), (2, 7), (3, 4), (5, 5)]):
+        want = TO.compute_signature(path, depth, None, None, windows)
+        G = randn(tuple(want.shape), seed=501)
+        got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[dtype]
+        assert rel_err(grad, TO.signature_vjp(path, G, depth, None, None, windows)) < TOL[dtype]
