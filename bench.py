@@ -6,6 +6,10 @@ One step = one forward + backward pass of the operator over one synthetic batch 
 resident in HBM.  The default workload is the headline configuration (depth-6 signature of 128
 Brownian paths with 1024 points in 4 dimensions, fp32).  Prints ONE JSON line.
 
+Before the W warm-up steps the step runs untimed for `--settle-ms` (default 1.5 s): an idle MI355X sits
+near 100 MHz and W steps of 0.15 ms end long before its shader clock has reached 2.4 GHz, so without
+this a short run times the ramp (measured: 0.161 ms per step after 100 steps, 0.139 ms in steady state).
+
 `roofline` is the fp32 (fp64 for f64 runs) vector-FMA roofline of the dominant call, the backward:
 algorithmic flops (2 per Horner node of the prefix closure of the requested words, per increment, x3
 for the backward) divided by its duration measured with HIP events on the launch stream.
@@ -26,8 +30,11 @@ import torch
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counters scaled on a
-# copy of known size (summaries and commands: profiles/dense_backward_kernel_c2.md, profiles/dense_kernels_c3_c5.md)
-TRAFFIC_BYTES = {("c2", "f32"): 50.0e6, ("c3", "f32"): 189.7e6, ("c5", "f32"): 57.7e6}
+# copy of known size (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00).  Summaries and commands:
+# profiles/dense_backward_kernel_c2.md, profiles/dense_kernels_c3_c5.md, profiles/batch_backward_kernel_c4.md.
+# c2, c4, c5: counters of the kernels as they are in this tree; c3: its kernel has not changed since its counters
+# were taken.  c4 counts the float atomics of the slab flush as written bytes (268 MB of the 377).
+TRAFFIC_BYTES = {("c2", "f32"): 50.0e6, ("c3", "f32"): 189.7e6, ("c4", "f32"): 377.4e6, ("c5", "f32"): 60.2e6}
 
 
 # ------------------------------------------------------------------------------------------------
@@ -214,6 +221,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-ms", type=float, default=1500.0,
+                    help="before the W warm-up steps, run untimed steps for this long so that the device has left "
+                         "its idle power state (its shader clock idles near 100 MHz and takes far longer than W short "
+                         "steps to reach 2.4 GHz); 0 switches it off")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -255,6 +266,13 @@ def main():
         out = mod(xg)
         torch.autograd.grad(out, xg, G)
 
+    # the device idles at a low shader clock: keep it busy until the clock has settled (untimed)
+    t_end = time.perf_counter() + args.settle_ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+
     # whole-step throughput: W warm-up steps, then exactly K steps between synchronisations
     def time_steps(fn):
         for _ in range(args.warmup):
@@ -278,6 +296,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
