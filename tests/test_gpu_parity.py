@@ -315,6 +315,12 @@ def test_sig_to_logsig_keep_cache(ps):
     g = randn(tuple(hyb.shape), seed=46)
     got = torch.ops.pathsig.logsig_backward_kept(logsig, cache, g.to(DEV), depth, True, words, sizes)
     assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
+    checks = ("test_schema", "test_faketensor", "test_autograd_registration")
+    sg = hyb.to(DEV).requires_grad_(True)
+    torch.library.opcheck(torch.ops.pathsig.sig_to_logsig_keep.default, (sg, depth, d, True, words, sizes),
+                          test_utils=checks)
+    torch.library.opcheck(torch.ops.pathsig.logsig_backward_kept.default,
+                          (logsig, cache, g.to(DEV), depth, True, words, sizes), test_utils=checks)
 
 
 @pytest.mark.parametrize("form", ["gather", "scatter"])
