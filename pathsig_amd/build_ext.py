@@ -20,7 +20,7 @@ TORCH_LIB = PKG / "libpathsig_torch.so"
 
 # (source, object, extra flags).  dense_kernels.hip is compiled once per group of register-tiled shapes and once
 # for the table of shapes and the dispatch, so the shapes build in parallel (the largest objects come first).
-DENSE_GROUPS = 4
+DENSE_GROUPS = 8  # kDenseGroups of csrc/dense.hpp
 UNITS = ([("dense_kernels.hip", f"dense_kernels_g{g}.o", [f"-DPSIG_GROUP={g}"]) for g in range(DENSE_GROUPS)]
          + [("batch_kernels.hip", "batch_kernels.o", []), ("words_kernels.hip", "words_kernels.o", []),
             ("logsig_kernels.hip", "logsig_kernels.o", []), ("dense_kernels.hip", "dense_kernels.o", []),

@@ -39,7 +39,7 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
 
 // The compiled shapes are dealt to kDenseGroups translation units (shape index modulo kDenseGroups); these are the
 // launch sequences of one group.  `bounds`: device array of letter bounds, or nullptr.
-constexpr int kDenseGroups = 4;
+constexpr int kDenseGroups = 8;
 template <int GROUP, typename T>
 hipError_t launch_dense_forward_group(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
                                       const int *bounds, T *keep, void *workspace, hipStream_t stream);

@@ -1241,20 +1241,41 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(20, 6, 2, 1, 1, 1) X(21, 7, 2, 1, 1, 1) X(22, 8, 2, 1, 1, 1) X(23, 2, 3, 2, 2, 1) X(24, 3, 3, 2, 2, 1) \
     X(25, 4, 3, 2, 2, 1) X(26, 5, 3, 2, 2, 1) X(27, 6, 3, 2, 2, 1) X(28, 7, 3, 2, 2, 1) X(29, 8, 3, 2, 2, 1) \
     X(30, 2, 4, 3, 3, 2) X(31, 3, 4, 3, 3, 2) X(32, 2, 5, 4, 4, 3) X(33, 2, 6, 4, 5, 4) X(34, 6, 6, 4, 4, 3) \
-    X(35, 7, 6, 4, 4, 3) X(36, 8, 6, 4, 4, 3)
+    X(35, 7, 6, 4, 4, 3) X(36, 8, 6, 4, 4, 3) X(37, 9, 2, 1, 1, 1) X(38, 10, 2, 1, 1, 1) \
+    X(39, 11, 2, 1, 1, 1) X(40, 12, 2, 1, 1, 1) X(41, 13, 2, 1, 1, 1) X(42, 14, 2, 1, 1, 1) \
+    X(43, 15, 2, 1, 1, 1) X(44, 16, 2, 1, 1, 1) X(45, 9, 3, 2, 2, 1) X(46, 10, 3, 2, 2, 1) \
+    X(47, 11, 3, 2, 2, 1) X(48, 12, 3, 2, 2, 1) X(49, 13, 3, 2, 2, 1) X(50, 14, 3, 2, 2, 1) \
+    X(51, 15, 3, 2, 2, 1) X(52, 16, 3, 2, 2, 1) X(53, 9, 4, 3, 3, 2) X(54, 10, 4, 3, 3, 2) \
+    X(55, 11, 4, 3, 3, 2) X(56, 12, 4, 3, 3, 2) X(57, 13, 4, 3, 3, 2) X(58, 14, 4, 3, 3, 2) \
+    X(59, 15, 4, 3, 3, 2) X(60, 16, 4, 3, 3, 2) X(61, 9, 5, 4, 4, 3) X(62, 10, 5, 4, 4, 3) \
+    X(63, 11, 5, 4, 4, 3) X(64, 12, 5, 4, 4, 3) X(65, 2, 7, 5, 6, 5) X(66, 3, 7, 4, 5, 4) \
+    X(67, 4, 7, 4, 5, 4) X(68, 3, 8, 5, 6, 5) X(69, 2, 9, 6, 8, 7) X(70, 2, 10, 6, 8, 7)
+
+// The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
+// two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.
+template <typename T, int D, int N, int PS>
+constexpr bool scan_fits() {
+    using GS = Geometry<D, N, PS>;
+    if (N < 3 || GS::kUnitBlocks > 1) return false;
+    const int64_t padded = RowStager<T, (int)GS::kLowSize, GS::kBlock>::kPadded;
+    return (2 * padded + 2 * GS::kLowSize) * (int64_t)sizeof(T) + 1024 <= 160 * 1024;
+}
 
 struct VariantInfo {
     int d, depth, block;  // block: threads of one unit
     int unit_blocks;      // blocks a unit is spread over (more than one: swept in one piece, dense only)
     int64_t sig_size, low_size;
-    bool bounds_ok;  // the sweeps can leave out top-level words by letter bounds
+    bool bounds_ok;       // the sweeps can leave out top-level words by letter bounds
+    bool chunks_ok[2];    // fp32, fp64: rows can be cut into time chunks
 };
 
-template <int D, int N, int P>
+template <int D, int N, int P, int PS>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
     return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
-                       LetterBounds<D, P>::kUsable && D <= 16};
+                       LetterBounds<D, P>::kUsable && D <= 16,
+                       {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
+                        G::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()}};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1275,7 +1296,7 @@ const int *stage_letter_bounds(const DenseChoice &dc, const int64_t *top_codes, 
 
 #endif
 
-#define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P>(),
+#define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P, PS>(),
 constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
 #undef PSIG_INFO
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -1420,9 +1441,9 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         profile_bracket(false, stream);
         return hipGetLastError();
     }
-    if constexpr (N < 3 || G::kUnitBlocks > 1) {
-        // depth 1 and 2 are never cut into time chunks (dense_choice): a row costs a few instructions per increment;
-        // nor are the shapes whose units take several blocks
+    if constexpr (G::kUnitBlocks > 1 || !scan_fits<T, D, N, PS>()) {
+        // never cut into time chunks (dense_choice): depth 1 and 2 (a row costs a few instructions per increment),
+        // shapes whose units take several blocks, rows too long for the scan kernel's LDS in this type
         return hipErrorNotSupported;
     } else {
         const int64_t units = rows * chunks;
@@ -1535,7 +1556,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
         }
-        if (v.unit_blocks > 1 && !all_dense) return dc;
+        const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
+        if (!chunks_ok && !all_dense) return dc;  // an embedded projection needs the time-chunked backward
         if (!all_dense) {
             // A word projection is worth computing densely when its top level keeps a fair share of the
             // words (the top level dominates the cost) and the dense rows fit comfortably in memory.
@@ -1550,8 +1572,9 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         }
         int chunks = pick_chunks(rows, v.block, L);
         if (const int64_t forced = options().chunks; forced >= 1 && forced <= 1024) chunks = (int)forced;
-        if (depth < 3) chunks = 1;  // the chunked backward needs a level below the top to scan over
-        if (v.unit_blocks > 1) chunks = 1;  // a row of such a shape is dozens of waves already
+        // not chunked: depth 1 and 2 (the chunked backward needs a level below the top to scan over), units of
+        // several blocks (a row is dozens of waves already), rows too long for the scan kernel's LDS
+        if (!chunks_ok) chunks = 1;
         if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
         dc.variant = i;
@@ -1569,6 +1592,17 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
     return dc;
 }
 
+// f(std::integral_constant<int, g>) for the group g of a shape
+template <int GI = 0, typename F>
+void dispatch_group(int group, F &&f) {
+    if constexpr (GI + 1 >= kDenseGroups) {
+        f(std::integral_constant<int, GI>{});
+    } else {
+        if (group == GI) f(std::integral_constant<int, GI>{});
+        else dispatch_group<GI + 1>(group, f);
+    }
+}
+
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
                                 const int64_t *top_codes, int64_t top_count, T *keep, void *workspace,
@@ -1577,12 +1611,11 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
     if (keep && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
-    switch (dc.variant % kDenseGroups) {
-        case 0: return launch_dense_forward_group<0, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
-        case 1: return launch_dense_forward_group<1, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
-        case 2: return launch_dense_forward_group<2, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
-        default: return launch_dense_forward_group<3, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
-    }
+    hipError_t e = hipErrorNotSupported;
+    dispatch_group(dc.variant % kDenseGroups, [&](auto g) {
+        e = launch_dense_forward_group<decltype(g)::value, T>(path, sig, shape, dc, bounds, keep, workspace, stream);
+    });
+    return e;
 }
 
 template <typename T>
@@ -1594,16 +1627,12 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
     if (kept && dc.keep_bytes == 0) return hipErrorInvalidValue;
     const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
                                             kVariants[dc.variant].depth, &workspace, stream);
-    switch (dc.variant % kDenseGroups) {
-#define PSIG_GROUP_CASE(GI)                                                                                          \
-    return launch_dense_backward_group<GI, T>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape, dc, bounds, \
-                                              kept, workspace, stream)
-        case 0: PSIG_GROUP_CASE(0);
-        case 1: PSIG_GROUP_CASE(1);
-        case 2: PSIG_GROUP_CASE(2);
-        default: PSIG_GROUP_CASE(3);
-#undef PSIG_GROUP_CASE
-    }
+    hipError_t e = hipErrorNotSupported;
+    dispatch_group(dc.variant % kDenseGroups, [&](auto g) {
+        e = launch_dense_backward_group<decltype(g)::value, T>(path, sig, grad_sig, grad_inc, grad_path, wrote_path,
+                                                               shape, dc, bounds, kept, workspace, stream);
+    });
+    return e;
 }
 
 #define PSIG_INSTANTIATE(T)                                                                                      \

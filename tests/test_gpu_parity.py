@@ -572,7 +572,8 @@ def test_gradcheck(ps):
 # shapes served by the register-tiled dense kernels (forward, backward, windows, long paths)
 # ------------------------------------------------------------------------------------------------
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5),
-         (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6)]
+         (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6),
+         (9, 2), (13, 2), (16, 2), (9, 3), (11, 3), (16, 3), (9, 4), (10, 4), (2, 7), (3, 7), (4, 7), (3, 8), (2, 9), (2, 10)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -763,7 +764,7 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
     elif case == "not_chunked":
         d, B, L, chunked = 4, 3000, 20, False
     elif case == "per_word":
-        d, B, L, chunked = 9, 3, 40, False          # no register-tiled shape for d = 9: per-word kernels, all dense
+        d, B, L, chunked = 17, 3, 40, False         # no register-tiled shape for d = 17: per-word kernels, all dense
     else:
         d, depth, L = 5, 5, 60
         B = 3 if case == "words_few_paths" else 20
@@ -788,7 +789,7 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
     grad_k = torch.ops.pathsig.signature_backward_kept(x, sig_k, G, chunks, *args)
     assert torch.equal(sig_k, sig)
     # two runs of the per-word backward differ by the order of their float atomics (a few 1e-6 of the largest
-    # gradient in fp32 at 6561 words); the register-tiled backward is deterministic without windows
+    # gradient in fp32 at 83521 words); the register-tiled backward is deterministic without windows
     close = TOL[dtype] * (0.5 if case == "per_word" else 0.1)
     assert rel_err(grad_k, grad) < close
     # the module takes the keeping pair when a gradient is wanted
@@ -851,11 +852,11 @@ def test_many_long_rows_fp32_one_chunk(ps, d, depth):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6)])
+@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6), (11, 4), (16, 4), (9, 5), (12, 5)])
 def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
-    """d^6 for d >= 6: a row's lanes (d^4 prefixes) do not fit one block; the unit is spread over two to four
-    blocks, swept in one piece, and the per-increment sums of the backward meet in memory.  With and without
-    windows (overlapping ones included)."""
+    """d^6 for d >= 6, d^4 for d >= 11, d^5 for d >= 9: a row's lanes (one per prefix) do not fit one block; the
+    unit is spread over two to twenty-one blocks, swept in one piece, and the per-increment sums of the backward
+    meet in memory.  With and without windows (overlapping ones included)."""
     B, L = 2, 8
     path = brownian_path(B, L, d, seed=500 + d) * 2.0
     for windows in (None, [(0, 8), (2, 7), (3, 4), (5, 5)]):

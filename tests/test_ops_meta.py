@@ -69,7 +69,7 @@ def test_chunk_buffer_size_follows_the_library():
     long_dense = _meta(128, 1024, 4)
     assert ops._chunks_numel(long_dense, 6, False, [], 0) % (128 * (4 + 16 + 64 + 256 + 1024)) == 0
     assert ops._chunks_numel(long_dense, 6, False, [], 0) > 0
-    assert ops._chunks_numel(_meta(128, 1024, 9), 4, False, [], 0) == 0      # no tiled shape for d = 9
+    assert ops._chunks_numel(_meta(128, 1024, 17), 4, False, [], 0) == 0     # no tiled shape for d = 17
     assert ops._chunks_numel(_meta(4096, 20, 4), 6, False, [], 0) == 0       # short paths, many rows: one chunk
 
 
