@@ -401,7 +401,10 @@ struct Geometry {
     // kUnitBlocks blocks (its lanes never talk to each other inside a sweep; the per-increment sums of the
     // backward then meet in memory).  Such shapes are swept in one piece, without time chunks.
     static constexpr int kUnitWaves = (kLanes + kWave - 1) / kWave;
-    static constexpr int kWaves = kUnitWaves < 16 ? kUnitWaves : 16;  // waves of one block
+    // waves of one block: sixteen at most, eight when the lane's sub-trie is large (a block of sixteen waves leaves
+    // each lane 128 registers, which the reverse sweep of such a shape overflows)
+    static constexpr int kMaxWaves = trie_size(D, N - P) > 40 ? 8 : 16;
+    static constexpr int kWaves = kUnitWaves < kMaxWaves ? kUnitWaves : kMaxWaves;
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
     static constexpr int kFwdSub = trie_size(D, N - P);    // sub-trie levels P+1..N
