@@ -207,7 +207,7 @@ __device__ __forceinline__ double row_total(double v) {
     return v;
 }
 
-// Sums of D values (D = 2, 4 or 8) over the 16 lanes of a DPP row, all at once: the first
+// Sums of D values (D = 2, 4, 8 or 16) over the 16 lanes of a DPP row, all at once: the first
 // log2(D) exchange steps halve the number of values a lane carries (a lane keeps the half selected by one
 // of its index bits and adds its partner's copy of that half), the remaining steps add single values.
 // Exchange partners are lane^1, lane^2, lane^8, lane^4, in that order.  Afterwards every lane holds the
@@ -1115,10 +1115,10 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int j = 0; j < P; ++j) my_cells[u[j] * G::kBlock] = T(0);
             }
-            if constexpr (kParts == 4 && D <= 8) {
+            if constexpr (kParts == 4 && D <= 16) {
                 // all letters in one pass of exchanges (the alphabet padded to a power of two with zeros);
                 // one store per row of 16 lanes
-                constexpr int DP = D <= 2 ? 2 : D <= 4 ? 4 : 8;
+                constexpr int DP = D <= 2 ? 2 : D <= 4 ? 4 : D <= 8 ? 8 : 16;
                 T padded[DP];
 #pragma unroll
                 for (int k = 0; k < DP; ++k) padded[k] = k < D ? tot[k] : T(0);
