@@ -980,14 +980,16 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
 }
 
 // LDS layout of the reverse sweep.  Per-increment sums leave a wave as four row sums; the tile flush adds the
-// parts of all waves in a fixed order.  The tile is shortened until the parts fit 48 KB of LDS.
+// parts of all waves in a fixed order.  The tile is shortened until the parts fit 48 KB of LDS (128 KB for the
+// widest alphabets, whose parts of sixteen increments would not fit a CU at all).
 template <typename T, int D, int N, int P>
 struct BackwardShape {
     using G = Geometry<D, N, P>;
     static constexpr int KS = N - P;
     static constexpr int kParts = 4;
     static constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
-    static constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32 : 16;
+    static constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32
+                                    : kRowBytes * 16 <= 131072 ? 16 : kRowBytes * 8 <= 131072 ? 8 : 4;
     static constexpr int kStage = kBwdTile * KS * D;
     static constexpr int kSums = G::kWaves * kParts;
     static constexpr int kSumRow = kBwdTile * D;
@@ -1115,16 +1117,19 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int j = 0; j < P; ++j) my_cells[u[j] * G::kBlock] = T(0);
             }
-            if constexpr (kParts == 4 && D <= 16) {
-                // all letters in one pass of exchanges (the alphabet padded to a power of two with zeros);
-                // one store per row of 16 lanes
+            if constexpr (kParts == 4) {
+                // up to sixteen letters in one pass of exchanges (padded to a power of two with zeros), wider
+                // alphabets sixteen letters at a time; one store per row of 16 lanes and pass
                 constexpr int DP = D <= 2 ? 2 : D <= 4 ? 4 : D <= 8 ? 8 : 16;
-                T padded[DP];
 #pragma unroll
-                for (int k = 0; k < DP; ++k) padded[k] = k < D ? tot[k] : T(0);
-                const T r = row_totals<T, DP>(padded, lane);
-                const int letter = row_letter<DP>(lane);
-                if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
+                for (int base = 0; base < D; base += DP) {
+                    T padded[DP];
+#pragma unroll
+                    for (int k = 0; k < DP; ++k) padded[k] = base + k < D ? tot[base + k] : T(0);
+                    const T r = row_totals<T, DP>(padded, lane);
+                    const int letter = base + row_letter<DP>(lane);
+                    if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
+                }
             } else {
 #pragma unroll
                 for (int k = 0; k < D; ++k) {
@@ -1252,7 +1257,15 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(55, 11, 4, 3, 3, 2) X(56, 12, 4, 3, 3, 2) X(57, 13, 4, 3, 3, 2) X(58, 14, 4, 3, 3, 2) \
     X(59, 15, 4, 3, 3, 2) X(60, 16, 4, 3, 3, 2) X(61, 9, 5, 4, 4, 3) X(62, 10, 5, 4, 4, 3) \
     X(63, 11, 5, 4, 4, 3) X(64, 12, 5, 4, 4, 3) X(65, 2, 7, 5, 6, 5) X(66, 3, 7, 4, 5, 4) \
-    X(67, 4, 7, 4, 5, 4) X(68, 3, 8, 5, 6, 5) X(69, 2, 9, 6, 8, 7) X(70, 2, 10, 6, 8, 7)
+    X(67, 4, 7, 4, 5, 4) X(68, 3, 8, 5, 6, 5) X(69, 2, 9, 6, 8, 7) X(70, 2, 10, 6, 8, 7) \
+    X(71, 17, 2, 1, 1, 1) X(72, 18, 2, 1, 1, 1) X(73, 19, 2, 1, 1, 1) X(74, 20, 2, 1, 1, 1) \
+    X(75, 21, 2, 1, 1, 1) X(76, 22, 2, 1, 1, 1) X(77, 23, 2, 1, 1, 1) X(78, 24, 2, 1, 1, 1) \
+    X(79, 25, 2, 1, 1, 1) X(80, 26, 2, 1, 1, 1) X(81, 27, 2, 1, 1, 1) X(82, 28, 2, 1, 1, 1) \
+    X(83, 29, 2, 1, 1, 1) X(84, 30, 2, 1, 1, 1) X(85, 31, 2, 1, 1, 1) X(86, 32, 2, 1, 1, 1) \
+    X(87, 17, 3, 2, 2, 1) X(88, 18, 3, 2, 2, 1) X(89, 19, 3, 2, 2, 1) X(90, 20, 3, 2, 2, 1) \
+    X(91, 21, 3, 2, 2, 1) X(92, 22, 3, 2, 2, 1) X(93, 23, 3, 2, 2, 1) X(94, 24, 3, 2, 2, 1) \
+    X(95, 25, 3, 2, 2, 1) X(96, 26, 3, 2, 2, 1) X(97, 27, 3, 2, 2, 1) X(98, 28, 3, 2, 2, 1) \
+    X(99, 29, 3, 2, 2, 1) X(100, 30, 3, 2, 2, 1) X(101, 31, 3, 2, 2, 1) X(102, 32, 3, 2, 2, 1)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.

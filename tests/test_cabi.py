@@ -83,10 +83,10 @@ def test_argument_errors_have_codes_and_messages(lib):
 
 def test_workspace_sizes(lib):
     # general kernels: the forward needs none, the backward one increment accumulator
-    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 17, 3, None, 0) == 0
-    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 17, 3, None, 0)
-    assert need >= 4 * 99 * 17 * 4
-    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 17, 3, None, 0) >= 4 * 99 * 17 * 8
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 33, 3, None, 0) == 0
+    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 33, 3, None, 0)
+    assert need >= 4 * 99 * 33 * 4
+    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 33, 3, None, 0) >= 4 * 99 * 33 * 8
     # a long path on a tiled shape is cut into chunks, which need scratch in the forward too
     assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, None, 0) > 0
     assert lib.pathsig_sig_forward_workspace(0, 4096, 64, 4, 6, None, 0) == 0

@@ -573,7 +573,8 @@ def test_gradcheck(ps):
 # ------------------------------------------------------------------------------------------------
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5),
          (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6),
-         (9, 2), (13, 2), (16, 2), (9, 3), (11, 3), (16, 3), (9, 4), (10, 4), (2, 7), (3, 7), (4, 7), (3, 8), (2, 9), (2, 10)]
+         (9, 2), (13, 2), (16, 2), (9, 3), (11, 3), (16, 3), (9, 4), (10, 4), (2, 7), (3, 7), (4, 7), (3, 8), (2, 9), (2, 10),
+         (17, 2), (32, 2), (17, 3), (27, 3), (32, 3)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
