@@ -197,12 +197,14 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
             set_error("workspace too small: need %zu bytes, got %zu", dc.forward_workspace, workspace_bytes);
             return PATHSIG_ERR_WORKSPACE;
         }
-        // a dense call writes straight into sig; an embedded projection goes through a dense buffer
-        T *dense = dc.embed ? (T *)workspace : (T *)sig;
+        // a dense call writes straight into sig; an embedded projection goes through a dense buffer (the buffer kept
+        // for the backward when that is the dense signature itself)
+        const bool keep_dense = dc.embed && dc.resweep && keep;
+        T *dense = keep_dense ? (T *)keep : dc.embed ? (T *)workspace : (T *)sig;
         void *rest = (unsigned char *)workspace + dc.dense_bytes;
         const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
-        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, top_codes, plan.size[depth], (T *)keep,
-                                               rest, stream);
+        hipError_t e = launch_dense_forward<T>((const T *)path, dense, shape, dc, top_codes, plan.size[depth],
+                                               dc.resweep ? (T *)nullptr : (T *)keep, rest, stream);
         if (e != hipSuccess) return launch_failed(e, "dense forward launch");
         if (dc.embed) {
             e = launch_gather_columns<T>(dense, (T *)sig, plan, d, codes, B * shape.W, stream);
@@ -247,21 +249,38 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     if (dc.usable) {
         unsigned char *extra = (unsigned char *)workspace + inc_bytes;
         const T *gdense = (const T *)grad_sig;
+        const T *sdense = (const T *)sig;
+        const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
+        size_t used = 0;
         if (dc.embed) {
-            // upstream gradient scattered into a zeroed dense buffer; the dense signature itself is not
-            // needed because the time-chunked backward rebuilds what it reads
+            // upstream gradient scattered into a zeroed dense buffer.  The time-chunked backward rebuilds what it
+            // reads of the dense signature; a shape that is swept in one piece reads the dense signature, which the
+            // forward kept or which is swept again here
             T *buf = (T *)extra;
+            used = dc.dense_bytes;
             e = launch_fill_zero<T>(buf, (int64_t)(dc.dense_bytes / sizeof(T)), stream);
             if (e != hipSuccess) return launch_failed(e, "fill launch");
             e = launch_scatter_columns<T>((const T *)grad_sig, buf, plan, d, codes, B * shape.W, stream);
             if (e != hipSuccess) return launch_failed(e, "scatter launch");
             gdense = buf;
+            sdense = nullptr;
+            if (dc.resweep) {
+                if (kept) {
+                    sdense = (const T *)kept;
+                } else {
+                    T *again = (T *)(extra + dc.dense_bytes);
+                    e = launch_dense_forward<T>((const T *)path, again, shape, dc, top_codes, plan.size[depth],
+                                                (T *)nullptr, extra + 2 * dc.dense_bytes, stream);
+                    if (e != hipSuccess) return launch_failed(e, "dense forward launch");
+                    sdense = again;
+                }
+                used = 2 * dc.dense_bytes;
+            }
         }
         bool wrote_path = false;
-        const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
-        e = launch_dense_backward<T>((const T *)path, dc.embed ? (const T *)nullptr : (const T *)sig, gdense, ginc,
-                                     (T *)grad_path, &wrote_path, shape, dc, top_codes, plan.size[depth],
-                                     (const T *)kept, extra + dc.dense_bytes, stream);
+        e = launch_dense_backward<T>((const T *)path, sdense, gdense, ginc, (T *)grad_path, &wrote_path, shape, dc,
+                                     top_codes, plan.size[depth], dc.resweep ? (const T *)nullptr : (const T *)kept,
+                                     extra + used, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
         if (wrote_path) return PATHSIG_OK;
     } else {

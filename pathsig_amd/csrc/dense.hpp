@@ -9,13 +9,16 @@ struct DenseChoice {
     bool usable;                // a register-tiled kernel exists for this call
     bool embed;                 // the call is a word projection that is computed densely and then gathered
     bool bounded;               // embed: the sweeps leave out top-level words by the letter bounds of the word list
+    bool resweep;               // embed with a shape that is not cut into time chunks: the backward needs the dense
+                                // signature, which the forward keeps or the backward computes again
     int variant;                // index into the table of compiled shapes
     int fwd_chunks;             // time chunks per (path, window) in the forward
     int bwd_chunks;             // ... and in the backward (at least 2 when embedding: no dense signature is saved)
     size_t dense_bytes;         // embed: bytes of one dense [rows, S] buffer
     size_t forward_workspace;   // bytes of scratch the forward needs (including the dense buffer)
     size_t backward_workspace;  // bytes of scratch the backward needs beyond the increment accumulator
-    size_t keep_bytes;          // bytes of chunk signatures the forward can keep for the backward (0: none)
+    size_t keep_bytes;          // bytes the forward can keep for the backward: chunk signatures, or (resweep) the
+                                // dense signature (0: none)
 };
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,

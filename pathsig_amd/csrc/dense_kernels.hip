@@ -1573,17 +1573,19 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
-        if (!chunks_ok && !all_dense) return dc;  // an embedded projection needs the time-chunked backward
         if (!all_dense) {
             // A word projection is worth computing densely when its top level keeps a fair share of the
-            // words (the top level dominates the cost) and the dense rows fit comfortably in memory.
-            if (!level_sizes || depth < 3) return dc;  // an embedded projection needs the time-chunked backward
+            // words (the top level dominates the cost) and the dense rows fit comfortably in memory.  The
+            // time-chunked backward rebuilds what it reads; for a shape that is not cut into chunks the backward
+            // needs the dense signature itself, kept by the forward or swept again (a second dense buffer).
+            if (!level_sizes) return dc;
             const int64_t top_dense = v.sig_size - v.low_size;
             if (level_sizes[depth] * 8 < top_dense) return dc;
-            if ((double)rows * (double)v.sig_size * (double)elem > 4e9) return dc;
+            if ((double)rows * (double)v.sig_size * (double)elem * (chunks_ok ? 1.0 : 2.0) > 4e9) return dc;
             dc.embed = true;
+            dc.resweep = !chunks_ok;
             dc.dense_bytes = pad256((size_t)rows * v.sig_size * elem);
-            dc.bounded = v.bounds_ok && level_sizes[depth] > 0 && level_sizes[depth] < top_dense &&
+            dc.bounded = chunks_ok && v.bounds_ok && level_sizes[depth] > 0 && level_sizes[depth] < top_dense &&
                          options().letter_bounds != 0;
         }
         int chunks = pick_chunks(rows, v.block, L);
@@ -1595,14 +1597,15 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         dc.usable = true;
         dc.variant = i;
         dc.fwd_chunks = chunks;
-        dc.bwd_chunks = (dc.embed && chunks < 2) ? 2 : chunks;
+        dc.bwd_chunks = (dc.embed && !dc.resweep && chunks < 2) ? 2 : chunks;
         dc.forward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
-        dc.backward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
+        dc.backward_workspace = (dc.resweep ? 2 : 1) * dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
         if (dc.fwd_chunks > 1) dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem);
         if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
         // the forward can hand its chunk signatures to the backward when both cut the rows the same way
         if (dc.bwd_chunks > 1 && dc.fwd_chunks == dc.bwd_chunks)
             dc.keep_bytes = (size_t)rows * dc.bwd_chunks * v.low_size * elem;
+        if (dc.resweep) dc.keep_bytes = (size_t)rows * v.sig_size * elem;
         return dc;
     }
     return dc;

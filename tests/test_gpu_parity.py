@@ -681,6 +681,46 @@ def test_projection_through_dense_kernels(ps, dtype, d, depth, kind):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,kind", [(3, 2, "lyndon"), (16, 2, "lyndon"), (20, 2, "dups"), (6, 6, "lyndon"),
+                                          (11, 4, "lyndon"), (9, 5, "words")])
+def test_projection_through_shapes_swept_in_one_piece(ps, dtype, d, depth, kind):
+    """Depth 2 and the shapes whose units take several blocks are never cut into time chunks, so the backward of
+    a projection computed through them reads the dense signature: kept by the forward (the modules) or swept
+    again (the stateless pair of operators).  Both must agree with the checker, with and without windows."""
+    B, L = 2, 9
+    if kind == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    elif kind == "dups":
+        top = random_word_set(d, depth, depth, 120, seed=21)
+        proj = ps.projections.words([(3,), (0,), (3,)] + top + top[:9], depth=depth, path_dim=d)
+    else:
+        top = random_word_set(d, depth, depth, d ** depth // 6, seed=22)
+        proj = ps.projections.words(random_word_set(d, 1, depth - 1, 50, seed=23) + top, depth=depth, path_dim=d)
+    sizes, codes = _plan(proj)
+    assert sizes[depth] * 8 >= d ** depth
+    path = brownian_path(B, L, d, seed=75) * 1.5
+    for windows in (None, [(0, 9), (2, 7), (4, 5), (6, 6), (2, 7)]):
+        want = TO.compute_signature(path, depth, sizes, codes, windows)
+        G = randn(tuple(want.shape), seed=76)
+        want_grad = TO.signature_vjp(path, G, depth, sizes, codes, windows)
+        got, grad = _run_sig(ps, path, depth, dtype, projection=proj, windows=windows, G=G)   # keeping pair
+        assert rel_err(got, want) < TOL[dtype]
+        assert rel_err(grad, want_grad) < TOL[dtype]
+        x = path.to(dtype).to(DEV)
+        win = None if windows is None else torch.tensor(windows, dtype=torch.int64, device=DEV)
+        mod = ps.Signature(depth=depth, projection=proj, windows=win)
+        args = (mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes, mod.use_windows,
+                mod._windows)
+        sig = torch.ops.pathsig.compute_signature(x, *args)
+        sig_k, kept = torch.ops.pathsig.compute_signature_keep(x, *args)
+        rows = B * (1 if windows is None else len(windows))
+        assert kept.numel() == rows * TO.dense_size(d, depth)      # the dense signature is what is kept
+        assert torch.equal(sig, sig_k)
+        g2 = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)            # sweeps again
+        assert rel_err(g2.cpu(), want_grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 def test_logsignature_lyndon_through_dense_kernels(ps, dtype):
     d, depth, B, L = 4, 4, 3, 60
     proj = ps.projections.lyndon(depth=depth, path_dim=d)
