@@ -97,6 +97,9 @@ int pathsig_sig_backward_noalloc(const void *path, const void *sig, const void *
  * skips the launch that would recompute them.  The per-word kernels hand over, in the same buffer, the
  * prefix values of the words whose prefixes are not all part of the signature (the backward otherwise
  * rebuilds them with a forward sweep, as src/pathsig/backward/sig_backward_kernels.cu:134-157 does).
+ * A word projection that is computed through a register-tiled shape which is swept in one piece (depth 2,
+ * shapes with more than 1024 lanes per row) hands over its dense signature, which the backward otherwise
+ * sweeps again.
  * pathsig_sig_chunks_bytes() returns the size of that buffer for a call, or 0 when the call has nothing to
  * hand over (then use the plain entry points).  All other arguments are as above; `chunks == NULL` makes
  * both functions identical to the plain ones.
