@@ -167,6 +167,10 @@ int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const vo
  *   "letter_bounds"   1 = embedded projections leave out unwanted top-level words (PATHSIG_NO_LETTER_BOUNDS sets 0)
  *   "logsig_scatter"  1 = the log-signature adjoint always takes its scatter form (PATHSIG_LOGSIG_SCATTER=1)
  *   "batch_tile"      cap on the increments per tile of the lanes-on-paths backward, 0 = none (PATHSIG_BATCH_TILE)
+ *   "embed_share"     which word projections run on the register-tiled kernels (dense sweep + gather of the
+ *                     wanted columns) instead of the per-word kernels: -1 = the library's rule (top level keeps
+ *                     1/8 of the dense one, or the dense sweep is estimated cheaper), 0 = none, n > 0 = those whose
+ *                     top level keeps at least 1/n of the dense one (PATHSIG_EMBED_SHARE)
  * Returns PATHSIG_ERR_ARGUMENT for an unknown name or a value out of range.
  */
 int pathsig_set_option(const char *name, int64_t value);

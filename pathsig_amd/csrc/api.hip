@@ -37,12 +37,13 @@ int64_t env_int(const char *name, int64_t fallback) {
 
 // Plain integers behind relaxed atomics: a setter on one thread and a call on another see whole values.
 struct OptionCells {
-    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile;
+    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share;
     OptionCells()
         : chunks(env_int("PATHSIG_CHUNKS", 0)),
           letter_bounds(getenv("PATHSIG_NO_LETTER_BOUNDS") ? 0 : 1),
           logsig_scatter(env_int("PATHSIG_LOGSIG_SCATTER", 0) == 1 ? 1 : 0),
-          batch_tile(env_int("PATHSIG_BATCH_TILE", 0)) {}
+          batch_tile(env_int("PATHSIG_BATCH_TILE", 0)),
+          embed_share(env_int("PATHSIG_EMBED_SHARE", -1)) {}
 };
 OptionCells &option_cells() {
     static OptionCells cells;  // the environment is read here, once
@@ -57,6 +58,7 @@ const Options &options() {
     snapshot.letter_bounds = c.letter_bounds.load(std::memory_order_relaxed);
     snapshot.logsig_scatter = c.logsig_scatter.load(std::memory_order_relaxed);
     snapshot.batch_tile = c.batch_tile.load(std::memory_order_relaxed);
+    snapshot.embed_share = c.embed_share.load(std::memory_order_relaxed);
     return snapshot;
 }
 
@@ -363,6 +365,8 @@ int pathsig_set_option(const char *name, int64_t value) {
         option_cells().logsig_scatter.store(value, std::memory_order_relaxed);
     } else if (!strcmp(name, "batch_tile") && value >= 0) {
         option_cells().batch_tile.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "embed_share") && value >= -1) {
+        option_cells().embed_share.store(value, std::memory_order_relaxed);
     } else {
         set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
         return PATHSIG_ERR_ARGUMENT;

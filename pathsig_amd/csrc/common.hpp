@@ -48,6 +48,8 @@ struct Options {
     int64_t letter_bounds;   // embedded projections leave out top-level words by letter bounds (default 1)
     int64_t logsig_scatter;  // log-signature adjoint in its scatter form even where the gather form fits (default 0)
     int64_t batch_tile;      // cap on the increments per tile of the lanes-on-paths backward (0: no cap)
+    int64_t embed_share;     // a projection runs on the register-tiled kernels when its top level keeps at least
+                             // 1/embed_share of the dense one (0: never; -1: the library's own rule)
 };
 const Options &options();
 

@@ -19,6 +19,7 @@
 // step (which yields H_{t-1} and dL/d(dx_t)), and keeps the top level of H equal to the upstream
 // gradient.  Adjoint values of the shared chain nodes stay lane-private partial sums (everything they
 // feed is linear in them), so the only cross-lane operation is the final sum of D numbers per step.
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
@@ -1574,13 +1575,31 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
         if (!all_dense) {
-            // A word projection is worth computing densely when its top level keeps a fair share of the
-            // words (the top level dominates the cost) and the dense rows fit comfortably in memory.  The
-            // time-chunked backward rebuilds what it reads; for a shape that is not cut into chunks the backward
-            // needs the dense signature itself, kept by the forward or swept again (a second dense buffer).
+            // A word projection is computed densely and gathered when that is the cheaper way: when its top level
+            // keeps a fair share of the dense one (the top level dominates the cost), or when the dense sweep is
+            // small against what the per-word kernels cost.  Those sweep the path one increment after the other
+            // whatever the number of words (about 1.7 us per increment), or about 4 ns per thousand (word, path,
+            // increment) when there are many; the dense kernels run at 40 TFLOP/s or more (25 for alphabets of more
+            // than eight letters; fp64: half) on 10 flops per signature coefficient, path and increment, and a
+            // step costs 80 us at least.
+            // The time-chunked backward rebuilds what it reads; for a shape that is not cut into chunks the
+            // backward needs the dense signature itself, kept by the forward or swept again (a second buffer).
             if (!level_sizes) return dc;
             const int64_t top_dense = v.sig_size - v.low_size;
-            if (level_sizes[depth] * 8 < top_dense) return dc;
+            const int64_t share = options().embed_share;
+            if (share == 0) return dc;
+            if (share > 0) {
+                if ((double)level_sizes[depth] * (double)share < (double)top_dense) return dc;
+            } else if (level_sizes[depth] * 8 < top_dense) {
+                double words = 0;
+                for (int k = 1; k <= depth; ++k) words += (double)level_sizes[k];
+                const double steps = (double)(L - 1);
+                const double per_word_us = std::max(1.7 * steps, 3.9e-6 * words * (double)rows * steps);
+                const double dense_us =
+                    std::max(80.0, 10.0 * (double)v.sig_size * (double)rows * steps / (v.d <= 8 ? 40e6 : 25e6) *
+                                       (elem == 8 ? 2.0 : 1.0));
+                if (dense_us > 0.8 * per_word_us) return dc;
+            }
             if ((double)rows * (double)v.sig_size * (double)elem * (chunks_ok ? 1.0 : 2.0) > 4e9) return dc;
             dc.embed = true;
             dc.resweep = !chunks_ok;

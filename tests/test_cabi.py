@@ -93,3 +93,24 @@ def test_workspace_sizes(lib):
     assert lib.pathsig_logsig_backward_workspace(0, 10, 3, 4, 81) >= 10 * (3 + 9 + 27) * 4 * 4
     # bad arguments give 0
     assert lib.pathsig_sig_forward_workspace(0, 4, 1, 5, 3, None, 0) == 0
+
+
+def test_sparse_projections_take_the_dense_kernels_when_that_is_cheaper(lib):
+    """A projection with a few words: the per-word kernels sweep the path one increment after the other, so on a
+    long path the dense kernels + a gather win as long as the dense signature is small; the forward then needs a
+    dense buffer as workspace.  (Host-side decision only; nothing is launched.)"""
+    import ctypes
+    def sizes(d, depth, top, low=3):
+        return (ctypes.c_int64 * (depth + 1))(0, *([low] * (depth - 1)), top)
+    dense = 4 * 128 * sum(4 ** k for k in range(1, 7))          # one fp32 dense row per path, d = 4, depth 6
+    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) >= dense
+    assert lib.pathsig_sig_forward_workspace(0, 128, 20, 4, 6, sizes(4, 6, 10), 0) == 0      # short path: per word
+    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 6, 6, sizes(6, 6, 10), 0) == 0    # 56 k coefficients: per word
+    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 33, 3, sizes(33, 3, 10), 0) == 0  # no compiled shape
+    try:
+        assert lib.pathsig_set_option(b"embed_share", 0) == 0
+        assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) == 0
+        assert lib.pathsig_set_option(b"embed_share", 10 ** 9) == 0
+        assert lib.pathsig_sig_forward_workspace(0, 128, 20, 4, 6, sizes(4, 6, 10), 0) >= dense
+    finally:
+        assert lib.pathsig_set_option(b"embed_share", -1) == 0

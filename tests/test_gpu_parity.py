@@ -93,8 +93,12 @@ def test_degenerate_windows_give_zero(ps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("route", ["share", "dense"])
 @pytest.mark.parametrize("kind", ["words", "lyndon", "gap", "all_words", "full_levels"])
-def test_projections(ps, dtype, kind):
+def test_projections(ps, set_option, dtype, kind, route):
+    """route "share": a projection runs on the register-tiled kernels only when its top level keeps 1/8 of the
+    dense one (the others exercise the per-word kernels); "dense": whenever a compiled shape exists."""
+    set_option("embed_share", 8 if route == "share" else 10 ** 9)
     d, depth, L, B = 3, 4, 15, 3
     if kind == "words":
         proj = ps.projections.words(random_word_set(d, 1, 4, 40, seed=5), depth=depth, path_dim=d)
@@ -121,10 +125,12 @@ def test_projections(ps, dtype, kind):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("route", ["share", "dense"])
 @pytest.mark.parametrize("B", [3, 20])
-def test_anisotropic_projection(ps, dtype, B):
+def test_anisotropic_projection(ps, set_option, dtype, B, route):
     """Weighted-degree truncation (`projections.py:132-223`): signature and log-signature through the projection,
     for a small batch (lanes on words) and a larger one (lanes on paths)."""
+    set_option("embed_share", 8 if route == "share" else 10 ** 9)
     d, depth, L = 4, 5, 16
     proj = ps.projections.anisotropic([1.0, 1.5, 2.0, 3.0], weight_threshold=5.0, depth=depth, path_dim=d)
     assert 0 < proj.sig_size < TO.dense_size(d, depth)
@@ -143,7 +149,9 @@ def test_anisotropic_projection(ps, dtype, B):
     assert rel_err(out, TO.logsignature(path, depth).index_select(-1, cols)) < TOL[dtype]
 
 
-def test_projection_with_windows(ps):
+@pytest.mark.parametrize("route", ["share", "dense"])
+def test_projection_with_windows(ps, set_option, route):
+    set_option("embed_share", 8 if route == "share" else 10 ** 9)
     d, depth, L, B = 4, 3, 20, 2
     proj = ps.projections.lyndon(depth=depth, path_dim=d)
     wins = [(0, 10), (5, 20), (7, 9)]
@@ -170,7 +178,8 @@ def test_projection_with_windows(ps):
     dict(d=40, depth=2, L=11, B=29, kind="dense"),
     dict(d=3, depth=7, L=12, B=50, kind="dups"),
 ])
-def test_projection_backward_lanes_on_paths(ps, dtype, case):
+def test_projection_backward_lanes_on_paths(ps, set_option, dtype, case):
+    set_option("embed_share", 8)    # sparse projections stay on the per-word kernels, whatever the path length
     d, depth, L, B, kind = case["d"], case["depth"], case["L"], case["B"], case["kind"]
     if kind == "words":
         proj = ps.projections.words(random_word_set(d, 1, depth, 45, seed=51), depth=depth, path_dim=d)
@@ -209,7 +218,8 @@ def test_projection_backward_lanes_on_paths(ps, dtype, case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-def test_projection_backward_lanes_on_paths_windows(ps, dtype):
+def test_projection_backward_lanes_on_paths_windows(ps, set_option, dtype):
+    set_option("embed_share", 8)
     d, depth, L, B = 4, 5, 30, 19
     proj = ps.projections.words(random_word_set(d, 2, 5, 60, seed=61), depth=depth, path_dim=d, full_levels=(1,))
     wins = [(0, 30), (3, 5), (2, 19), (15, 30), (4, 6), (0, 2), (28, 30), (5, 25), (5, 25), (7, 8), (40, 50)]
@@ -790,6 +800,7 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
     on words for a few paths, lanes on paths for a dozen and more); the buffer is empty when neither applies."""
     import ctypes
     from pathsig_amd import _load
+    set_option("embed_share", 8)    # the words_* cases are about the per-word kernels
     depth, kw, chunked = 4, {}, True
     if case == "dense":
         d, B, L = 4, 5, 300

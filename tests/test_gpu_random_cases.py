@@ -67,6 +67,9 @@ def test_random_signature_cases(set_option, seed):
         if d ** depth > 40000:
             continue
         set_option("chunks", int(chunks) if chunks else 0)
+        # projections: through the register-tiled kernels only with 1/8 of the top level kept (the rest on the
+        # per-word kernels), or whenever a compiled shape exists
+        set_option("embed_share", 8 if case % 2 == 0 else 10 ** 9)
         sizes, codes = (None, None) if proj is None else (proj.level_sizes, proj._codes)
         path = brownian_path(B, L, d, seed=seeds[0]) * scale
         want = TO.compute_signature(path, depth, sizes, codes, windows)
