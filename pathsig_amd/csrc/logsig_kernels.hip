@@ -261,29 +261,45 @@ struct MatvecShape {
     int64_t bb, sb, sn;       // strides of B
 };
 
-// bval(b, k, m) supplies the B operand (strides bb, sb, sn of the shape are not used by this form)
-template <typename T, typename BVal, typename Store>
-__device__ void block_matvec_fn(const T *A, BVal &&bval, const MatvecShape &sh, T *red, Store &&store) {
-    const int64_t outputs = sh.nb * sh.no;
+// Counts fit 32 bits (the caller's layouts are bounded by the workspace limits); the operands are walked with
+// pointers that advance by a constant, so the inner loop is two loads, one multiply-add and two pointer steps.
+template <typename T, typename Store>
+__device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *red, Store &&store) {
+    const int no = (int)sh.no, nk = (int)sh.nk, nm = (int)sh.nm;
+    const int outputs = (int)sh.nb * no;
     int parts = 1;
-    while ((int64_t)parts * 2 * outputs <= kLogBlock && (int64_t)parts * 2 <= sh.nk) parts *= 2;
+    while (parts * 2 * outputs <= kLogBlock && parts * 2 <= nk) parts *= 2;
     const int slots = kLogBlock / parts;  // outputs worked on at once; >= outputs whenever parts > 1
     const bool k_fast = sh.sk < sh.so;
     const int tid = threadIdx.x;
     const int part = k_fast ? tid % parts : tid / slots;
     const int oloc = k_fast ? tid / parts : tid % slots;
-    for (int64_t o0 = 0; o0 < outputs; o0 += slots) {
-        const int64_t oo = o0 + oloc;
-        const int64_t bi = oo / sh.no, o = oo - bi * sh.no;
+    const int64_t astep = (int64_t)parts * sh.sk, bstep = (int64_t)parts * sh.sb;
+    for (int o0 = 0; o0 < outputs; o0 += slots) {
+        const int oo = o0 + oloc;
+        const int bi = oo / no, o = oo - bi * no;
         T acc = T(0);
         if (oo < outputs) {
-            const T *a = A + bi * sh.ab + o * sh.so;
-            if (sh.nm == 1) {
-#pragma unroll 16
-                for (int64_t k = part; k < sh.nk; k += parts) acc += a[k * sh.sk] * bval(bi, k, (int64_t)0);
+            const T *ap = A + (int64_t)bi * sh.ab + (int64_t)o * sh.so + (int64_t)part * sh.sk;
+            const T *bp = B + (int64_t)bi * sh.bb + (int64_t)part * sh.sb;
+            if (nm == 1) {
+#pragma unroll 8
+                for (int k = part; k < nk; k += parts) {
+                    acc += *ap * *bp;
+                    ap += astep;
+                    bp += bstep;
+                }
             } else {
-                for (int64_t k = part; k < sh.nk; k += parts)
-                    for (int64_t m = 0; m < sh.nm; ++m) acc += a[k * sh.sk + m * sh.sm] * bval(bi, k, m);
+                for (int k = part; k < nk; k += parts) {
+                    const T *am = ap, *bm = bp;
+                    for (int m = 0; m < nm; ++m) {
+                        acc += *am * *bm;
+                        am += sh.sm;
+                        bm += sh.sn;
+                    }
+                    ap += astep;
+                    bp += bstep;
+                }
             }
         }
         if (parts > 1) {
@@ -292,21 +308,15 @@ __device__ void block_matvec_fn(const T *A, BVal &&bval, const MatvecShape &sh, 
             if (part == 0 && oo < outputs) {
                 T total = T(0);
                 for (int q = 0; q < parts; ++q) total += red[k_fast ? oloc * parts + q : q * slots + oloc];
-                store(bi, o, total);
+                store((int64_t)bi, (int64_t)o, total);
             }
             __syncthreads();
         } else if (oo < outputs) {
-            store(bi, o, acc);
+            store((int64_t)bi, (int64_t)o, acc);
         }
     }
     __threadfence_block();
     __syncthreads();
-}
-
-template <typename T, typename Store>
-__device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *red, Store &&store) {
-    block_matvec_fn<T>(A, [&](int64_t bi, int64_t k, int64_t m) { return B[bi * sh.bb + k * sh.sb + m * sh.sn]; }, sh, red,
-                       store);
 }
 
 // Top-level part of the gather form, one block per (row, split, side): with the top-level gradient g as a
@@ -531,7 +541,9 @@ LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, in
     const bool listed = top_size != width;
     // the dense copy of the top-level gradient must stay modest: 1 GiB
     const bool fits = (double)rows * (double)width * (double)elem <= 1073741824.0;
-    if (depth >= 2 && !forced_scatter && (!listed || fits) && rows > 0) {
+    // the gather form counts its products in 32 bits
+    const bool small = (double)width * (double)depth < 2e9;
+    if (depth >= 2 && !forced_scatter && (!listed || fits) && small && rows > 0) {
         lp.gather = true;
         lp.q_elems = 2 * rows * lower;  // R and Q
         lp.top_elems = listed ? rows * width : 0;
