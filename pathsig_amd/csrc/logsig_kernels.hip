@@ -372,15 +372,14 @@ __global__ void logsig_q_kernel(const T *__restrict__ cache, T *__restrict__ Q_a
 }
 
 // Levels below the top, one block per row, going down.  `a` ([lower columns][depth]) holds a_k: in LDS when the
-// launch provides room for it (a_in_lds; the kernel is a chain of short dependent passes over `a`, so their
+// launch provides room for it (A_IN_LDS; the kernel is a chain of short dependent passes over `a`, so their
 // latency is what it costs), else in the workspace.  `R` ([lower columns], workspace) are the top-level sums of
 // logsig_gather_top_kernel, which has also stored the top-level part of the gradient in grad_sig.
-template <typename T>
+template <typename T, bool A_IN_LDS>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ logsig,
                                                                   const T *__restrict__ cache,
                                                                   const T *__restrict__ grad_logsig, T *grad_sig,
-                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp,
-                                                                  int a_in_lds) {
+                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp) {
     extern __shared__ __align__(16) unsigned char gather_smem[];
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
@@ -389,7 +388,10 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     const T *Cr = cache + row * hp.total * N;
     const T *gl = grad_logsig + row * hp.total;
     T *gs = grad_sig + row * hp.total;
-    T *a = a_in_lds ? reinterpret_cast<T *>(gather_smem) : a_all + row * hp.lower * N;
+    // the address space of `a` is fixed at compile time, so that its loads are LDS loads and not generic ones
+    T *a;
+    if constexpr (A_IN_LDS) a = reinterpret_cast<T *>(gather_smem);
+    else a = a_all + row * hp.lower * N;
     const T *R = R_all + row * hp.lower;
     int64_t width[kMaxDepth + 1];  // d^k
     width[0] = 1;
@@ -397,15 +399,17 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
 
     // a_k(w) starts from its top-level part, sum_v a_{k+1}(w v) L(v) = -f_{k+1} R(w); the top-level columns
     // of the gradient are g
+    __shared__ T invf[kMaxDepth + 2];  // 1 / k!
+    if (threadIdx.x == 0) {
+        invf[0] = invf[1] = T(1);
+        for (int k = 2; k <= N + 1; ++k) invf[k] = invf[k - 1] / T(k);
+    }
+    __syncthreads();
     for (int n = 1; n < N; ++n) {
         for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
             const int64_t col = hp.off[n] + i;
             const T r = R[col];
-            T f = T(1);
-            for (int m = 1; m <= N; ++m) {
-                f /= T(m + 1);  // 1 / (m + 1)!
-                a[col * N + m - 1] = m <= n ? -f * r : T(0);
-            }
+            for (int m = 1; m <= N; ++m) a[col * N + m - 1] = m <= n ? -invf[m + 1] * r : T(0);
         }
     }
     for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) gs[hp.off[N] + i] = gl[hp.off[N] + i];
@@ -431,11 +435,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
         for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
             const T lam = gl[hp.off[n] + i] + an[i * N] + gsn[i];
             gsn[i] = lam;
-            T f = T(1);
-            for (int k = 2; k <= n; ++k) {
-                f /= T(k);
-                an[i * N + k - 1] -= f * lam;
-            }
+            for (int k = 2; k <= n; ++k) an[i * N + k - 1] -= invf[k] * lam;
         }
         __threadfence_block();
         __syncthreads();
@@ -594,13 +594,18 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
         // the adjoint of the cache goes to LDS when a block's share of it fits beside the static arrays
         const size_t a_bytes = (size_t)hp.lower * (size_t)depth * sizeof(T);
         const bool a_in_lds = a_bytes <= 144 * 1024;
-        if (a_in_lds && a_bytes > 32 * 1024) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_kernel<T>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)a_bytes);
-            if (e != hipSuccess) return e;
+        if (a_in_lds) {
+            if (a_bytes > 32 * 1024) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_kernel<T, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)a_bytes);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL((logsig_gather_kernel<T, true>), dim3((unsigned)rows), dim3(kLogBlock), a_bytes, stream,
+                               logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
+        } else {
+            hipLaunchKernelGGL((logsig_gather_kernel<T, false>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, logsig,
+                               cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
         }
-        hipLaunchKernelGGL(logsig_gather_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), a_in_lds ? a_bytes : 0, stream,
-                           logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp, a_in_lds ? 1 : 0);
         return hipGetLastError();
     }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
