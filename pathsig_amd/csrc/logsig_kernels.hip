@@ -350,6 +350,43 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *_
     }
 }
 
+// The same products for many rows of a small layout, one block per row: the row's top-level gradient is built
+// once in LDS as a dense d^N array (a listed top level is scattered into it, repeated words adding up) and all
+// 2 (N - 1) products read it from there.  With thousands of rows the launch over (row, split, side) above is
+// bound by reading each row's dense gradient 2 (N - 1) times from L2, and needs that array in memory first.
+template <typename T>
+__global__ void __launch_bounds__(kLogBlock) logsig_gather_top_rows_kernel(
+    const T *__restrict__ logsig, const T *__restrict__ Q_all, const T *__restrict__ grad_logsig, T *grad_sig,
+    T *R_all, HybridPlan hp, const int64_t *__restrict__ top_words, int64_t top_dense) {
+    extern __shared__ __align__(16) unsigned char top_smem[];
+    __shared__ T red[kLogBlock];
+    T *gtop = reinterpret_cast<T *>(top_smem);
+    const int N = hp.depth;
+    const int64_t row = blockIdx.x;
+    const T *lgs = logsig + row * hp.total;
+    const T *gl = grad_logsig + row * hp.total + hp.off[N];
+    if (hp.size[N] != top_dense) {  // a listed top level (possibly empty)
+        for (int64_t i = threadIdx.x; i < top_dense; i += kLogBlock) gtop[i] = T(0);
+        __syncthreads();
+        for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) atomicAdd(&gtop[top_words[i]], gl[i]);
+    } else {
+        for (int64_t i = threadIdx.x; i < top_dense; i += kLogBlock) gtop[i] = gl[i];
+    }
+    __syncthreads();
+    int64_t wj = 1, wi = top_dense;
+    for (int j = 1; j < N; ++j) {
+        wj *= hp.d;
+        wi /= hp.d;
+        const int i = N - j;
+        T *R = R_all + row * hp.lower + hp.off[j];
+        block_matvec<T>(gtop, lgs + hp.off[i], MatvecShape{1, wj, wi, 1, 0, wi, 1, 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) { R[o] = r; });
+        T *gsi = grad_sig + row * hp.total + hp.off[i];
+        block_matvec<T>(gtop, Q_all + row * hp.lower + hp.off[j], MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, 1, 0}, red,
+                        [&](int64_t, int64_t o, T r) { gsi[o] = r; });
+    }
+}
+
 // Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! for every column below the top, all rows
 template <typename T>
 __global__ void logsig_q_kernel(const T *__restrict__ cache, T *__restrict__ Q_all, HybridPlan hp, int64_t rows) {
@@ -562,24 +599,6 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
     T *gradP = workspace;
     if (lp.gather) {
         T *R = gradP + lp.a_elems;
-        const T *gtop = grad_logsig + hp.off[depth];
-        int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
-        if (lp.top_elems > 0) {
-            T *dense = R + lp.q_elems;
-            hipError_t e = launch_fill_zero<T>(dense, lp.top_elems, stream);
-            if (e != hipSuccess) return e;
-            const int64_t n = rows * top_size;
-            if (n > 0) {
-                int64_t blocks = (n + 255) / 256;
-                if (blocks > 65536) blocks = 65536;
-                hipLaunchKernelGGL(scatter_top_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_logsig, dense,
-                                   hp, top_words, rows, lp.top_dense);
-                e = hipGetLastError();
-                if (e != hipSuccess) return e;
-            }
-            gtop = dense;
-            top_stride = lp.top_dense;
-        }
         T *Q = R + rows * hp.lower;
         {
             int64_t blocks = (rows * hp.lower + 255) / 256;
@@ -587,9 +606,42 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
             if (blocks < 1) blocks = 1;
             hipLaunchKernelGGL(logsig_q_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, cache, Q, hp, rows);
         }
-        hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2), dim3(kLogBlock), 0,
-                           stream, logsig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
         hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        // top-level products: with many rows of a small layout one block per row with the row's dense top-level
+        // gradient in LDS; else one block per (row, split, side) over a dense copy of that gradient in memory
+        const size_t top_bytes = (size_t)lp.top_dense * sizeof(T);
+        if (rows >= 256 && top_bytes <= 64 * 1024) {
+            if (top_bytes > 32 * 1024) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_top_rows_kernel<T>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)top_bytes);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), top_bytes, stream,
+                               logsig, (const T *)Q, grad_logsig, grad_sig, R, hp, top_words, lp.top_dense);
+        } else {
+            const T *gtop = grad_logsig + hp.off[depth];
+            int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
+            if (lp.top_elems > 0) {
+                T *dense = R + lp.q_elems;
+                e = launch_fill_zero<T>(dense, lp.top_elems, stream);
+                if (e != hipSuccess) return e;
+                const int64_t n = rows * top_size;
+                if (n > 0) {
+                    int64_t blocks = (n + 255) / 256;
+                    if (blocks > 65536) blocks = 65536;
+                    hipLaunchKernelGGL(scatter_top_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_logsig,
+                                       dense, hp, top_words, rows, lp.top_dense);
+                    e = hipGetLastError();
+                    if (e != hipSuccess) return e;
+                }
+                gtop = dense;
+                top_stride = lp.top_dense;
+            }
+            hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2),
+                               dim3(kLogBlock), 0, stream, logsig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
+        }
+        e = hipGetLastError();
         if (e != hipSuccess) return e;
         // the adjoint of the cache goes to LDS when a block's share of it fits beside the static arrays
         const size_t a_bytes = (size_t)hp.lower * (size_t)depth * sizeof(T);

@@ -372,6 +372,41 @@ def test_logsig_adjoint_both_forms(ps, set_option, form, dtype, d, depth, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,top", [
+    (3, 4, [5, 80, 17, 17, 2]),      # listed top level, unsorted, with a repeated word
+    (2, 6, None),                      # dense top level
+    (4, 5, "lyndon"),
+    (7, 3, []),                        # empty top level
+    (6, 5, "lyndon"),                  # 7776 dense top-level words: 30 KB (fp32), 61 KB (fp64) of LDS per row
+])
+def test_logsig_adjoint_many_rows(ps, dtype, d, depth, top):
+    """From 256 rows on, a layout whose dense top level fits 64 KB takes the top-level products of the adjoint
+    from the row's gradient staged in LDS (one block per row); same checks as for a few rows."""
+    rows = 300
+    if top == "lyndon":
+        proj = ps.projections.lyndon(depth=depth, path_dim=d)
+        top = list(proj._codes[-proj.level_sizes[depth]:])
+    path = brownian_path(rows, 7, d, seed=77) * 1.5
+    dense = TO.signature(path, depth)
+    n_top = d ** depth if top is None else len(top)
+    cols = TO.hybrid_columns(d, depth, n_top, top)
+    hyb = dense[:, cols]
+    sizes = [0] + [d ** k for k in range(1, depth)] + [n_top]
+    words = torch.tensor([] if top is None else top, dtype=torch.int64, device=DEV)
+    alt = top is not None
+    g = randn(tuple(hyb.shape), seed=78)
+    logsig, cache = torch.ops.pathsig.sig_to_logsig_keep(hyb.to(dtype).to(DEV), depth, d, alt, words, sizes)
+    got = torch.ops.pathsig.logsig_backward_kept(logsig, cache, g.to(dtype).to(DEV), depth, alt, words, sizes)
+    sub = slice(0, rows, 7)
+    want = TO.logsig_vjp(hyb[sub], g[sub], depth, d, n_top, top)
+    assert rel_err(got[sub], want) < TOL[dtype]
+    # the same rows a few at a time take the other kernel; both must agree closely
+    few = torch.ops.pathsig.logsig_backward_kept(logsig[:40].contiguous(), cache[:40].contiguous(),
+                                                 g[:40].to(dtype).to(DEV), depth, alt, words, sizes)
+    assert rel_err(got[:40], few) < TOL[dtype] * 0.1
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("d,depth,L,scale,kind", [
     (2, 7, 3, 2.0, "lyndon"), (2, 8, 3, 2.0, "lyndon"), (2, 8, 65, 2.0, "dense"), (2, 8, 130, 2.0, "dense"),
     (2, 8, 130, 2.0, "lyndon"), (3, 6, 2, 2.0, "dense"), (3, 6, 200, 2.0, "dense"), (3, 7, 40, 2.0, "lyndon"),
