@@ -33,7 +33,15 @@ namespace psig {
 
 namespace {
 
-constexpr int kLogBlock = 512;
+constexpr int kLogBlock = 512;  // threads of a block at most; the kernels take their stride from blockDim.x
+
+// Threads per row (a row is one block).  A few rows get the largest block: the time of one row is all there is.
+// With many rows of a small layout most of 512 threads would idle through every pass while few rows fit a CU, so
+// the block shrinks with the layout and more rows run side by side.
+inline int logsig_block(int64_t columns, int64_t rows) {
+    if (rows <= 256 || columns > 2048) return kLogBlock;
+    return columns > 512 ? 256 : columns > 128 ? 128 : 64;
+}
 
 struct HybridPlan {
     int depth;
@@ -65,7 +73,7 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
     const bool listed = (DEG == depth) && hp.top_is_list;
     const T *right = STABLE ? lg : s;
     // the blocks of one row (gridDim.y of them) share the words of the level
-    for (int64_t i = (int64_t)blockIdx.y * kLogBlock + threadIdx.x; i < hp.size[DEG]; i += (int64_t)gridDim.y * kLogBlock) {
+    for (int64_t i = (int64_t)blockIdx.y * (int)blockDim.x + threadIdx.x; i < hp.size[DEG]; i += (int64_t)gridDim.y * (int)blockDim.x) {
         const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
         // dense column of every proper prefix, right factor of every proper suffix
         uint64_t pidx[DEG + 1];
@@ -170,7 +178,7 @@ __device__ void logsig_backward_level(const T *__restrict__ lgrow, const T *__re
     const uint64_t d = (uint64_t)hp.d;
     const bool top = (DEG == depth);
     const bool listed = top && hp.top_is_list;
-    for (int64_t i = threadIdx.x; i < hp.size[DEG]; i += kLogBlock) {
+    for (int64_t i = threadIdx.x; i < hp.size[DEG]; i += (int)blockDim.x) {
         const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
         uint64_t pidx[DEG + 1], sidx[DEG + 1];
         {
@@ -226,9 +234,9 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
     sink.lds_gP = sink.lds_gs + lds_cols;
     sink.lds_cols = lds_cols;
     sink.depth = hp.depth;
-    for (int64_t i = threadIdx.x; i < hp.total; i += kLogBlock) sink.gs[i] = T(0);
-    for (int64_t i = threadIdx.x; i < hp.lower * hp.depth; i += kLogBlock) sink.gP[i] = T(0);
-    for (int64_t i = threadIdx.x; i < lds_cols * (hp.depth + 1); i += kLogBlock) sink.lds_gs[i] = T(0);
+    for (int64_t i = threadIdx.x; i < hp.total; i += (int)blockDim.x) sink.gs[i] = T(0);
+    for (int64_t i = threadIdx.x; i < hp.lower * hp.depth; i += (int)blockDim.x) sink.gP[i] = T(0);
+    for (int64_t i = threadIdx.x; i < lds_cols * (hp.depth + 1); i += (int)blockDim.x) sink.lds_gs[i] = T(0);
     __threadfence_block();
     __syncthreads();
     for (int deg = hp.depth; deg >= 1; --deg) {
@@ -243,7 +251,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
         __threadfence_block();
         __syncthreads();
     }
-    for (int64_t i = threadIdx.x; i < lds_cols; i += kLogBlock) sink.gs[i] = sink.lds_gs[i];
+    for (int64_t i = threadIdx.x; i < lds_cols; i += (int)blockDim.x) sink.gs[i] = sink.lds_gs[i];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -268,8 +276,8 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
     const int no = (int)sh.no, nk = (int)sh.nk, nm = (int)sh.nm;
     const int outputs = (int)sh.nb * no;
     int parts = 1;
-    while (parts * 2 * outputs <= kLogBlock && parts * 2 <= nk) parts *= 2;
-    const int slots = kLogBlock / parts;  // outputs worked on at once; >= outputs whenever parts > 1
+    while (parts * 2 * outputs <= (int)blockDim.x && parts * 2 <= nk) parts *= 2;
+    const int slots = (int)blockDim.x / parts;  // outputs worked on at once; >= outputs whenever parts > 1
     const bool k_fast = sh.sk < sh.so;
     const int tid = threadIdx.x;
     const int part = k_fast ? tid % parts : tid / slots;
@@ -366,11 +374,11 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_rows_kernel(
     const T *lgs = logsig + row * hp.total;
     const T *gl = grad_logsig + row * hp.total + hp.off[N];
     if (hp.size[N] != top_dense) {  // a listed top level (possibly empty)
-        for (int64_t i = threadIdx.x; i < top_dense; i += kLogBlock) gtop[i] = T(0);
+        for (int64_t i = threadIdx.x; i < top_dense; i += (int)blockDim.x) gtop[i] = T(0);
         __syncthreads();
-        for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) atomicAdd(&gtop[top_words[i]], gl[i]);
+        for (int64_t i = threadIdx.x; i < hp.size[N]; i += (int)blockDim.x) atomicAdd(&gtop[top_words[i]], gl[i]);
     } else {
-        for (int64_t i = threadIdx.x; i < top_dense; i += kLogBlock) gtop[i] = gl[i];
+        for (int64_t i = threadIdx.x; i < top_dense; i += (int)blockDim.x) gtop[i] = gl[i];
     }
     __syncthreads();
     int64_t wj = 1, wi = top_dense;
@@ -443,13 +451,13 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     }
     __syncthreads();
     for (int n = 1; n < N; ++n) {
-        for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
+        for (int64_t i = threadIdx.x; i < width[n]; i += (int)blockDim.x) {
             const int64_t col = hp.off[n] + i;
             const T r = R[col];
             for (int m = 1; m <= N; ++m) a[col * N + m - 1] = m <= n ? -invf[m + 1] * r : T(0);
         }
     }
-    for (int64_t i = threadIdx.x; i < hp.size[N]; i += kLogBlock) gs[hp.off[N] + i] = gl[hp.off[N] + i];
+    for (int64_t i = threadIdx.x; i < hp.size[N]; i += (int)blockDim.x) gs[hp.off[N] + i] = gl[hp.off[N] + i];
     __threadfence_block();
     __syncthreads();
 
@@ -469,7 +477,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
                             [&](int64_t, int64_t o, T r) { gsn[o] += r; });
         }
         // lam(w) = g(w) + a_1(w) + the sums above is the gradient of the word; a_k(w) -= lam(w) / k! for k >= 2
-        for (int64_t i = threadIdx.x; i < width[n]; i += kLogBlock) {
+        for (int64_t i = threadIdx.x; i < width[n]; i += (int)blockDim.x) {
             const T lam = gl[hp.off[n] + i] + an[i * N] + gsn[i];
             gsn[i] = lam;
             for (int k = 2; k <= n; ++k) an[i * N + k - 1] -= invf[k] * lam;
@@ -530,18 +538,19 @@ template <typename T, bool STABLE>
 hipError_t forward_pass(const T *sig, T *logsig, T *C, const HybridPlan &hp, int64_t rows, int64_t top_size,
                         const int64_t *top_words, hipStream_t stream) {
     const int depth = hp.depth;
-    int64_t slices = (top_size + 4 * kLogBlock - 1) / (4 * kLogBlock);
+    const int blk = logsig_block(hp.total, rows);
+    int64_t slices = (top_size + 4 * blk - 1) / (4 * blk);
     if (slices > 16) slices = 16;
     if (depth < 2 || slices < 2) {
-        hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig,
+        hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(blk), 0, stream, sig,
                            logsig, C, hp, top_words, 1, depth);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, sig, logsig,
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(blk), 0, stream, sig, logsig,
                        C, hp, top_words, 1, depth - 1);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows, (unsigned)slices), dim3(kLogBlock), 0,
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows, (unsigned)slices), dim3(blk), 0,
                        stream, sig, logsig, C, hp, top_words, depth, depth);
     return hipGetLastError();
 }
@@ -596,6 +605,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
     if (rows <= 0) return hipSuccess;
     const HybridPlan hp = make_hybrid(d, depth, top_size, top_words);
     const LogsigBackwardPlan lp = logsig_backward_plan(sizeof(T), rows, d, depth, top_size);
+    const int blk = logsig_block(hp.total, rows);
     T *gradP = workspace;
     if (lp.gather) {
         T *R = gradP + lp.a_elems;
@@ -617,7 +627,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)top_bytes);
                 if (e != hipSuccess) return e;
             }
-            hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), top_bytes, stream,
+            hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(blk), top_bytes, stream,
                                logsig, (const T *)Q, grad_logsig, grad_sig, R, hp, top_words, lp.top_dense);
         } else {
             const T *gtop = grad_logsig + hp.off[depth];
@@ -652,17 +662,17 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)a_bytes);
                 if (e != hipSuccess) return e;
             }
-            hipLaunchKernelGGL((logsig_gather_kernel<T, true>), dim3((unsigned)rows), dim3(kLogBlock), a_bytes, stream,
+            hipLaunchKernelGGL((logsig_gather_kernel<T, true>), dim3((unsigned)rows), dim3(blk), a_bytes, stream,
                                logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
         } else {
-            hipLaunchKernelGGL((logsig_gather_kernel<T, false>), dim3((unsigned)rows), dim3(kLogBlock), 0, stream, logsig,
+            hipLaunchKernelGGL((logsig_gather_kernel<T, false>), dim3((unsigned)rows), dim3(blk), 0, stream, logsig,
                                cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
         }
         return hipGetLastError();
     }
     const int64_t lds_cols = lds_columns(d, depth, sizeof(T), 32 * 1024);
     const size_t lds_bytes = (size_t)lds_cols * (size_t)(depth + 1) * sizeof(T);
-    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(kLogBlock), lds_bytes, stream, logsig, cache,
+    hipLaunchKernelGGL(logsig_backward_kernel<T>, dim3((unsigned)rows), dim3(blk), lds_bytes, stream, logsig, cache,
                        grad_logsig, grad_sig, gradP, hp, top_words, lds_cols);
     return hipGetLastError();
 }
