@@ -95,6 +95,9 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
         const uint64_t own = (uint64_t)(hp.off[DEG] + i);
         const T sw = s[own];
         T *Cw = C + own * (uint64_t)depth;
+        // the Q form never reads the cache rows of the top level (nothing is longer than a top-level word), so
+        // they are not written: for many rows the cache is most of what this kernel moves
+        const bool keep_row = !STABLE || DEG < depth;
         T acc = sw;
 #pragma unroll
         for (int m = 2; m <= DEG; ++m) {
@@ -102,11 +105,12 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
 #pragma unroll
             for (int k = m - 1; k < DEG; ++k) pv += C[pidx[k] * (uint64_t)depth + (uint64_t)(m - 2)] * sufv[DEG - k];
             if constexpr (STABLE) acc -= inv_factorial<T>(m) * pv;
-            Cw[m - 1] = pv;
+            if (keep_row) Cw[m - 1] = pv;
         }
-        for (int m = DEG + 1; m <= depth; ++m) Cw[m - 1] = T(0);
+        if (keep_row)
+            for (int m = DEG + 1; m <= depth; ++m) Cw[m - 1] = T(0);
         if constexpr (STABLE) {
-            Cw[0] = acc;
+            if (keep_row) Cw[0] = acc;
             lg[own] = acc;
         } else {
             Cw[0] = sw;

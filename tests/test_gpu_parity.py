@@ -306,8 +306,9 @@ def test_sig_to_logsig_cache_layout(ps):
 
 def test_sig_to_logsig_keep_cache(ps):
     """The keeping forward returns the same log-signature and, as its cache, the tensor powers of that
-    log-signature (entry k - 1 of a word's row: its coefficient in L^(x)k); the kept backward agrees with the
-    checker's adjoint."""
+    log-signature for the words below the top level (entry k - 1 of a word's row: its coefficient in L^(x)k;
+    the adjoint never reads the rows of top-level words, which are left unwritten); the kept backward agrees
+    with the checker's adjoint."""
     d, depth, B = 3, 4, 2
     top = [5, 80, 17, 17, 2]
     path = brownian_path(B, 9, d, seed=45) * 1.5
@@ -321,7 +322,8 @@ def test_sig_to_logsig_keep_cache(ps):
     logsig, cache = torch.ops.pathsig.sig_to_logsig_keep(hyb.to(DEV), depth, d, True, words, sizes)
     assert cache.shape == (B, len(cols) * depth)
     assert rel_err(logsig, want_log) < 1e-12
-    assert rel_err(cache, want_cache) < 1e-12
+    low = (len(cols) - len(top)) * depth       # the rows of the top level are not part of the hand-over
+    assert rel_err(cache[:, :low], want_cache[:, :low]) < 1e-12
     g = randn(tuple(hyb.shape), seed=46)
     got = torch.ops.pathsig.logsig_backward_kept(logsig, cache, g.to(DEV), depth, True, words, sizes)
     assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
