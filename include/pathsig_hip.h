@@ -148,8 +148,9 @@ int pathsig_logsig_backward(const void *sig, const void *P, const void *grad_log
  * The same pair with a hand-over from the forward to the backward (no counterpart in the reference).  The
  * forward writes, instead of P, the cache its own adjoint reads: cache [rows, S * depth] with
  * cache[idx * depth + (k - 1)] = level-|w| part of (log S)^(x)k at word idx (entry 0 is the log-signature
- * itself), 0 for k > |w|, for the words below the top level; the rows of top-level words are not written
- * (the adjoint never reads them).  The backward takes that cache and the log-signature and skips rebuilding them.
+ * itself) for the words below the top level; entry |w| of such a row holds -sum_{m<=|w|} (log S)^(x)m (w) / (m+1)!
+ * (the weight of w as a prefix in the adjoint's top-level sums), later entries 0; the rows of top-level words are
+ * not written (the adjoint never reads them).  The backward takes that cache and the log-signature and skips rebuilding them.
  */
 int pathsig_logsig_forward_keep(const void *sig, void *logsig, void *cache, int dtype, int64_t rows, int64_t d,
                                 int depth, int64_t top_size, const int64_t *top_words, void *stream);

@@ -248,7 +248,11 @@ def logsig_power_cache(logsig_hybrid: torch.Tensor, depth: int, d: int, top_size
                        top_codes: Optional[Sequence[int]] = None) -> torch.Tensor:
     """Cache of the keeping forward (`pathsig_logsig_forward_keep`; no counterpart in the reference): with
     L = log S, cache[..., idx * depth + (k - 1)] = level-|w| part of L^(x)k at word idx (entry 0 is L itself),
-    zero for k above the word's length.  Built here from plain truncated tensor products of L."""
+    zero for k above the word's length, except that a word w below the top level carries in entry |w|
+    (k = |w| + 1) the sum -sum_{m=1}^{|w|} (L^(x)m)(w) / (m + 1)!, the weight with which w enters the top-level
+    sums of the adjoint as a prefix.  Built here from plain truncated tensor products of L.  (The library leaves
+    the rows of top-level words unwritten; here they hold the powers.)"""
+    import math
     offs = dense_level_offsets(d, depth)
     if top_size is None:
         top_size = d ** depth
@@ -264,7 +268,11 @@ def logsig_power_cache(logsig_hybrid: torch.Tensor, depth: int, d: int, top_size
     colt = torch.tensor(cols, dtype=torch.int64)
     Q = [torch.cat(pw, dim=-1).index_select(-1, colt) for pw in powers]
     Q[0] = logsig_hybrid
-    return torch.stack(Q, dim=-1).reshape(*lead, -1)
+    out = torch.stack(Q, dim=-1).clone()                       # [..., S, depth]
+    for n in range(1, depth):                                   # words of length n < depth: entry n
+        lo, hi = offs[n], offs[n + 1]
+        out[..., lo:hi, n] = -sum(Q[m - 1][..., lo:hi] / math.factorial(m + 1) for m in range(1, n + 1))
+    return out.reshape(*lead, -1)
 
 
 # ----------------------------------------------------------------------------------------------

@@ -99,20 +99,29 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
         // they are not written: for many rows the cache is most of what this kernel moves
         const bool keep_row = !STABLE || DEG < depth;
         T acc = sw;
+        T qc = T(0);  // -sum_{m=2}^{DEG} Q_m(w) / (m + 1)!
 #pragma unroll
         for (int m = 2; m <= DEG; ++m) {
             T pv = T(0);
 #pragma unroll
             for (int k = m - 1; k < DEG; ++k) pv += C[pidx[k] * (uint64_t)depth + (uint64_t)(m - 2)] * sufv[DEG - k];
-            if constexpr (STABLE) acc -= inv_factorial<T>(m) * pv;
+            if constexpr (STABLE) {
+                acc -= inv_factorial<T>(m) * pv;
+                qc -= inv_factorial<T>(m + 1) * pv;
+            }
             if (keep_row) Cw[m - 1] = pv;
         }
-        if (keep_row)
-            for (int m = DEG + 1; m <= depth; ++m) Cw[m - 1] = T(0);
         if constexpr (STABLE) {
-            if (keep_row) Cw[0] = acc;
+            if (keep_row) {
+                // entry |w| of the row, which no product reads: Qc(w) = -sum_{m=1}^{|w|} Q_m(w) / (m + 1)!, the
+                // weight with which w enters the top-level sums of the adjoint as a prefix
+                Cw[0] = acc;
+                Cw[DEG] = qc - inv_factorial<T>(2) * acc;
+                for (int m = DEG + 2; m <= depth; ++m) Cw[m - 1] = T(0);
+            }
             lg[own] = acc;
         } else {
+            for (int m = DEG + 1; m <= depth; ++m) Cw[m - 1] = T(0);
             Cw[0] = sw;
         }
     }
@@ -334,11 +343,11 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
 // Top-level part of the gather form, one block per (row, split, side): with the top-level gradient g as a
 // d^j x d^(N-j) matrix, side 0 computes R(u) = sum_v g(uv) L(v) for the prefixes u of length j, side 1
 // computes T(v) = sum_u g(uv) Qc(u) for the suffixes v of length N - j, where
-// Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! comes from logsig_q_kernel.  R goes to its own workspace array, T
+// Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! is entry |u| of u's cache row (the forward puts it there).  R goes to its own workspace array, T
 // initialises the gradient.
 template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *__restrict__ logsig,
-                                                                      const T *__restrict__ Q_all,
+                                                                      const T *__restrict__ cache,
                                                                       const T *__restrict__ gtop_all, T *grad_sig,
                                                                       T *R_all, HybridPlan hp, int64_t top_dense) {
     __shared__ T red[kLogBlock];
@@ -357,7 +366,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *_
                         [&](int64_t, int64_t o, T r) { R[o] = r; });
     } else {
         T *gsi = grad_sig + row * hp.total + hp.off[i];
-        block_matvec<T>(gtop, Q_all + row * hp.lower + hp.off[j], MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, 1, 0}, red,
+        block_matvec<T>(gtop, cache + (row * hp.total + hp.off[j]) * N + j, MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, N, 0}, red,
                         [&](int64_t, int64_t o, T r) { gsi[o] = r; });
     }
 }
@@ -368,7 +377,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *_
 // bound by reading each row's dense gradient 2 (N - 1) times from L2, and needs that array in memory first.
 template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_rows_kernel(
-    const T *__restrict__ logsig, const T *__restrict__ Q_all, const T *__restrict__ grad_logsig, T *grad_sig,
+    const T *__restrict__ logsig, const T *__restrict__ cache, const T *__restrict__ grad_logsig, T *grad_sig,
     T *R_all, HybridPlan hp, const int64_t *__restrict__ top_words, int64_t top_dense) {
     extern __shared__ __align__(16) unsigned char top_smem[];
     __shared__ T red[kLogBlock];
@@ -394,29 +403,8 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_rows_kernel(
         block_matvec<T>(gtop, lgs + hp.off[i], MatvecShape{1, wj, wi, 1, 0, wi, 1, 0, 0, 1, 0}, red,
                         [&](int64_t, int64_t o, T r) { R[o] = r; });
         T *gsi = grad_sig + row * hp.total + hp.off[i];
-        block_matvec<T>(gtop, Q_all + row * hp.lower + hp.off[j], MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, 1, 0}, red,
+        block_matvec<T>(gtop, cache + (row * hp.total + hp.off[j]) * N + j, MatvecShape{1, wi, wj, 1, 0, 1, wi, 0, 0, N, 0}, red,
                         [&](int64_t, int64_t o, T r) { gsi[o] = r; });
-    }
-}
-
-// Qc(u) = -sum_{k=2}^{|u|+1} Q_{k-1}(u) / k! for every column below the top, all rows
-template <typename T>
-__global__ void logsig_q_kernel(const T *__restrict__ cache, T *__restrict__ Q_all, HybridPlan hp, int64_t rows) {
-    const int N = hp.depth;
-    const int64_t total = rows * hp.lower;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t row = idx / hp.lower, col = idx - row * hp.lower;
-        int n = 1;
-        while (n + 1 < N && col >= hp.off[n + 1]) ++n;
-        const T *Cc = cache + (row * hp.total + col) * N;
-        T q = T(0);
-        T f = T(1);
-        for (int k = 2; k <= n + 1; ++k) {
-            f /= T(k);
-            q -= f * Cc[k - 2];
-        }
-        Q_all[idx] = q;
     }
 }
 
@@ -595,7 +583,7 @@ LogsigBackwardPlan logsig_backward_plan(size_t elem, int64_t rows, int64_t d, in
     const bool small = (double)width * (double)depth < 2e9;
     if (depth >= 2 && !forced_scatter && (!listed || fits) && small && rows > 0) {
         lp.gather = true;
-        lp.q_elems = 2 * rows * lower;  // R and Q
+        lp.q_elems = rows * lower;  // R
         lp.top_elems = listed ? rows * width : 0;
     }
     return lp;
@@ -613,15 +601,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
     T *gradP = workspace;
     if (lp.gather) {
         T *R = gradP + lp.a_elems;
-        T *Q = R + rows * hp.lower;
-        {
-            int64_t blocks = (rows * hp.lower + 255) / 256;
-            if (blocks > 65536) blocks = 65536;
-            if (blocks < 1) blocks = 1;
-            hipLaunchKernelGGL(logsig_q_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, cache, Q, hp, rows);
-        }
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        hipError_t e = hipSuccess;
         // top-level products: with many rows of a small layout one block per row with the row's dense top-level
         // gradient in LDS; else one block per (row, split, side) over a dense copy of that gradient in memory
         const size_t top_bytes = (size_t)lp.top_dense * sizeof(T);
@@ -632,7 +612,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(blk), top_bytes, stream,
-                               logsig, (const T *)Q, grad_logsig, grad_sig, R, hp, top_words, lp.top_dense);
+                               logsig, cache, grad_logsig, grad_sig, R, hp, top_words, lp.top_dense);
         } else {
             const T *gtop = grad_logsig + hp.off[depth];
             int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
@@ -653,7 +633,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                 top_stride = lp.top_dense;
             }
             hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2),
-                               dim3(kLogBlock), 0, stream, logsig, (const T *)Q, gtop, grad_sig, R, hp, top_stride);
+                               dim3(kLogBlock), 0, stream, logsig, cache, gtop, grad_sig, R, hp, top_stride);
         }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
