@@ -133,4 +133,7 @@ def test_logsignature_entry_points(lib, dtype):
     torch.cuda.synchronize()
     tol = TOL[dtype]
     assert rel_err(logsig, want_log) < tol and rel_err(P, want_P) < tol and rel_err(grad, want_grad) < tol
-    assert torch.equal(logsig_k, logsig) and rel_err(cache, want_cache) < tol and rel_err(grad_k, want_grad) < tol
+    low = (hyb.shape[-1] - len(top)) * depth          # the cache rows of the top-level words are not written
+    assert torch.isnan(cache[:, low:]).all()
+    assert torch.equal(logsig_k, logsig) and rel_err(cache[:, :low], want_cache[:, :low]) < tol
+    assert rel_err(grad_k, want_grad) < tol
