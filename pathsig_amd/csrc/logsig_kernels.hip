@@ -453,23 +453,92 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     __threadfence_block();
     __syncthreads();
 
+    const int BLK = (int)blockDim.x, tid = (int)threadIdx.x;
     for (int n = N - 1; n >= 1; --n) {
         T *an = a + hp.off[n] * N;
         T *gsn = gs + hp.off[n];
-        // a_k(w) += sum_v a_{k+1}(w v) L(v) over the levels between this one and the top, all k in one batch
-        for (int i = 1; n + i < N; ++i) {
-            block_matvec<T>(a + hp.off[n + i] * N + 1, lgs + hp.off[i],
-                            MatvecShape{n, width[n], width[i], 1, 1, width[i] * N, N, 0, 0, 1, 0}, red,
-                            [&](int64_t bi, int64_t o, T r) { an[o * N + bi] += r; });
-        }
-        // gradient += sum_u sum_{k=2}^{|u|+1} a_k(u w) Q_{k-1}(u) over the same levels
-        for (int j = 1; n + j < N; ++j) {
-            block_matvec<T>(a + hp.off[n + j] * N + 1, Cr + hp.off[j] * N,
-                            MatvecShape{1, width[n], width[j], j, 0, N, width[n] * N, 1, 0, N, 1}, red,
-                            [&](int64_t, int64_t o, T r) { gsn[o] += r; });
+        const int wn = (int)width[n];
+        const int levels = N - 1 - n;  // levels between this one and the top
+        if (levels > 0) {
+            const int longest = (int)width[levels];
+            // a_k(w) += sum_v a_{k+1}(w v) L(v), v over all those levels at once, k = 1..n (output = (k, w)).
+            // When there are fewer outputs than threads, `parts` threads share an output (lanes along v, which
+            // is contiguous in a) and their partial sums meet in LDS.
+            {
+                const int outputs = n * wn;
+                int parts = 1;
+                while (parts * 2 * outputs <= BLK && parts * 2 <= longest) parts *= 2;
+                const int slots = BLK / parts, part = tid % parts, oloc = tid / parts;
+                for (int o0 = 0; o0 < outputs; o0 += slots) {
+                    const int oo = o0 + oloc;
+                    const int bi = oo / wn, o = oo - bi * wn;
+                    T acc = T(0);
+                    if (oo < outputs) {
+                        for (int i = 1; i <= levels; ++i) {
+                            const int wi = (int)width[i];
+                            const T *ap = a + (hp.off[n + i] + (int64_t)o * wi + part) * N + 1 + bi;
+                            const T *bp = lgs + hp.off[i] + part;
+                            for (int k = part; k < wi; k += parts) {
+                                acc += *ap * *bp;
+                                ap += (int64_t)parts * N;
+                                bp += parts;
+                            }
+                        }
+                    }
+                    if (parts > 1) {
+                        red[tid] = acc;
+                        __syncthreads();
+                        if (part == 0 && oo < outputs) {
+                            T total = T(0);
+                            for (int q = 0; q < parts; ++q) total += red[oloc * parts + q];
+                            an[o * N + bi] += total;
+                        }
+                        __syncthreads();
+                    } else if (oo < outputs) {
+                        an[o * N + bi] += acc;
+                    }
+                }
+            }
+            // gradient(w) += sum_u sum_{k=2}^{|u|+1} a_k(u w) Q_{k-1}(u), u over the same levels (output = w; lanes
+            // along w, which is contiguous in a; the parts of an output split the range of u)
+            {
+                int parts = 1;
+                while (parts * 2 * wn <= BLK && parts * 2 <= longest) parts *= 2;
+                const int slots = BLK / parts, part = tid / slots, oloc = tid % slots;
+                for (int o0 = 0; o0 < wn; o0 += slots) {
+                    const int o = o0 + oloc;
+                    T acc = T(0);
+                    if (o < wn) {
+                        for (int j = 1; j <= levels; ++j) {
+                            const int wj = (int)width[j];
+                            const T *ap = a + (hp.off[n + j] + (int64_t)part * wn + o) * N + 1;
+                            const T *bp = Cr + (hp.off[j] + part) * N;
+                            for (int k = part; k < wj; k += parts) {
+                                for (int m = 0; m < j; ++m) acc += ap[m] * bp[m];
+                                ap += (int64_t)parts * wn * N;
+                                bp += (int64_t)parts * N;
+                            }
+                        }
+                    }
+                    if (parts > 1) {
+                        red[tid] = acc;
+                        __syncthreads();
+                        if (part == 0 && o < wn) {
+                            T total = T(0);
+                            for (int q = 0; q < parts; ++q) total += red[q * slots + oloc];
+                            gsn[o] += total;
+                        }
+                        __syncthreads();
+                    } else if (o < wn) {
+                        gsn[o] += acc;
+                    }
+                }
+            }
+            __threadfence_block();
+            __syncthreads();
         }
         // lam(w) = g(w) + a_1(w) + the sums above is the gradient of the word; a_k(w) -= lam(w) / k! for k >= 2
-        for (int64_t i = threadIdx.x; i < width[n]; i += (int)blockDim.x) {
+        for (int i = tid; i < wn; i += BLK) {
             const T lam = gl[hp.off[n] + i] + an[i * N] + gsn[i];
             gsn[i] = lam;
             for (int k = 2; k <= n; ++k) an[i * N + k - 1] -= invf[k] * lam;
