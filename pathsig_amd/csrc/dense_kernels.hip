@@ -1266,7 +1266,15 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(87, 17, 3, 2, 2, 1) X(88, 18, 3, 2, 2, 1) X(89, 19, 3, 2, 2, 1) X(90, 20, 3, 2, 2, 1) \
     X(91, 21, 3, 2, 2, 1) X(92, 22, 3, 2, 2, 1) X(93, 23, 3, 2, 2, 1) X(94, 24, 3, 2, 2, 1) \
     X(95, 25, 3, 2, 2, 1) X(96, 26, 3, 2, 2, 1) X(97, 27, 3, 2, 2, 1) X(98, 28, 3, 2, 2, 1) \
-    X(99, 29, 3, 2, 2, 1) X(100, 30, 3, 2, 2, 1) X(101, 31, 3, 2, 2, 1) X(102, 32, 3, 2, 2, 1)
+    X(99, 29, 3, 2, 2, 1) X(100, 30, 3, 2, 2, 1) X(101, 31, 3, 2, 2, 1) X(102, 32, 3, 2, 2, 1) \
+    X(103, 33, 2, 1, 1, 1) X(104, 34, 2, 1, 1, 1) X(105, 35, 2, 1, 1, 1) X(106, 36, 2, 1, 1, 1) \
+    X(107, 37, 2, 1, 1, 1) X(108, 38, 2, 1, 1, 1) X(109, 39, 2, 1, 1, 1) X(110, 40, 2, 1, 1, 1) \
+    X(111, 41, 2, 1, 1, 1) X(112, 42, 2, 1, 1, 1) X(113, 43, 2, 1, 1, 1) X(114, 44, 2, 1, 1, 1) \
+    X(115, 45, 2, 1, 1, 1) X(116, 46, 2, 1, 1, 1) X(117, 47, 2, 1, 1, 1) X(118, 48, 2, 1, 1, 1) \
+    X(119, 49, 2, 1, 1, 1) X(120, 50, 2, 1, 1, 1) X(121, 51, 2, 1, 1, 1) X(122, 52, 2, 1, 1, 1) \
+    X(123, 53, 2, 1, 1, 1) X(124, 54, 2, 1, 1, 1) X(125, 55, 2, 1, 1, 1) X(126, 56, 2, 1, 1, 1) \
+    X(127, 57, 2, 1, 1, 1) X(128, 58, 2, 1, 1, 1) X(129, 59, 2, 1, 1, 1) X(130, 60, 2, 1, 1, 1) \
+    X(131, 61, 2, 1, 1, 1) X(132, 62, 2, 1, 1, 1) X(133, 63, 2, 1, 1, 1) X(134, 64, 2, 1, 1, 1)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.

@@ -171,11 +171,11 @@ def test_projection_with_windows(ps, set_option, route):
 @pytest.mark.parametrize("case", [
     dict(d=3, depth=4, L=15, B=13, kind="words"),
     dict(d=3, depth=4, L=40, B=37, kind="gap"),
-    dict(d=5, depth=3, L=23, B=64, kind="dense"),
+    dict(d=33, depth=3, L=23, B=64, kind="dense"),      # no register-tiled shape: all levels dense, per word
     dict(d=16, depth=6, L=19, B=33, kind="c4"),
     dict(d=2, depth=12, L=9, B=17, kind="long"),
     dict(d=7, depth=5, L=70, B=24, kind="full_low"),
-    dict(d=40, depth=2, L=11, B=29, kind="dense"),
+    dict(d=70, depth=2, L=11, B=29, kind="dense"),      # wider than any register-tiled shape
     dict(d=3, depth=7, L=12, B=50, kind="dups"),
 ])
 def test_projection_backward_lanes_on_paths(ps, set_option, dtype, case):
@@ -621,7 +621,7 @@ def test_gradcheck(ps):
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5),
          (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6),
          (9, 2), (13, 2), (16, 2), (9, 3), (11, 3), (16, 3), (9, 4), (10, 4), (2, 7), (3, 7), (4, 7), (3, 8), (2, 9), (2, 10),
-         (17, 2), (32, 2), (17, 3), (27, 3), (32, 3)]
+         (17, 2), (32, 2), (17, 3), (27, 3), (32, 3), (33, 2), (50, 2), (64, 2)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])

@@ -18,7 +18,8 @@ DEV = "cuda"
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (8, 5), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5)]
 OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6), (6, 3), (9, 4), (12, 2),
          (11, 4), (20, 3), (3, 8), (2, 10), (27, 2),        # tiled: several blocks per unit, wide, deep
-         (33, 2), (2, 11), (35, 3)]                           # no tiled shape: per-word kernels
+         (45, 2),                                            # tiled, widest kind
+         (70, 2), (2, 11), (35, 3)]                           # no tiled shape: per-word kernels
 
 
 def _random_case(rng, ps):
