@@ -980,6 +980,30 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     }
 }
 
+// Depth 2: the signature of a chunk below the top level is its level 1, the sum of its increments.  One block
+// per (row, chunk); zero_rows as in dense_forward_kernel (the block also clears the points of its chunk in a
+// [B, L, d] buffer, the last chunk of a row the final point too).
+template <typename T>
+__global__ void __launch_bounds__(kWave) chunk_level1_kernel(const T *__restrict__ path, T *__restrict__ chunk_low,
+                                                             SigShape shape, int chunks, T *__restrict__ zero_rows) {
+    const int64_t unit = blockIdx.x;
+    const int64_t row = unit / chunks;
+    const int c = (int)(unit - row * chunks);
+    const int64_t b = row / shape.W, w = row - b * shape.W;
+    const Span span = unit_span(shape, w);
+    int64_t begin, end;
+    chunk_range(span.steps, chunks, c, begin, end);
+    const int64_t d = shape.d;
+    const T *x = path + (b * shape.L + span.start) * d;
+    for (int64_t a = threadIdx.x; a < d; a += kWave)
+        chunk_low[unit * d + a] = end > begin ? x[end * d + a] - x[begin * d + a] : T(0);
+    if (zero_rows) {
+        const int64_t points = end - begin + (c == chunks - 1 ? 1 : 0);
+        T *z = zero_rows + (b * shape.L + span.start + begin) * d;
+        for (int64_t idx = threadIdx.x; idx < points * d; idx += kWave) z[idx] = T(0);
+    }
+}
+
 // LDS layout of the reverse sweep.  Per-increment sums leave a wave as four row sums; the tile flush adds the
 // parts of all waves in a fixed order.  The tile is shortened until the parts fit 48 KB of LDS (128 KB for the
 // widest alphabets, whose parts of sixteen increments would not fit a CU at all).
@@ -1281,7 +1305,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 template <typename T, int D, int N, int PS>
 constexpr bool scan_fits() {
     using GS = Geometry<D, N, PS>;
-    if (N < 3 || GS::kUnitBlocks > 1) return false;
+    if (N < 2 || GS::kUnitBlocks > 1) return false;
     const int64_t padded = RowStager<T, (int)GS::kLowSize, GS::kBlock>::kPadded;
     return (2 * padded + 2 * GS::kLowSize) * (int64_t)sizeof(T) + 1024 <= 160 * 1024;
 }
@@ -1467,8 +1491,8 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         return hipGetLastError();
     }
     if constexpr (G::kUnitBlocks > 1 || !scan_fits<T, D, N, PS>()) {
-        // never cut into time chunks (dense_choice): depth 1 and 2 (a row costs a few instructions per increment),
-        // shapes whose units take several blocks, rows too long for the scan kernel's LDS in this type
+        // never cut into time chunks (dense_choice): shapes whose units take several blocks, rows too long for
+        // the scan kernel's LDS in this type
         return hipErrorNotSupported;
     } else {
         const int64_t units = rows * chunks;
@@ -1485,10 +1509,15 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             // chunk signatures below the top level: the depth N-1 forward kernel on the same units
             // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
             // (the forward kernel needs a prefix shorter than its depth; the layout it writes does not depend on it)
-            constexpr int PK = P <= N - 2 ? P : N - 2;
-            hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, PK, 1>), dim3((unsigned)units),
-                               dim3(Geometry<D, N - 1, PK>::kBlock), 0, stream, path, chunk_low, shape, chunks,
-                               accumulate ? (T *)nullptr : grad_path);
+            if constexpr (N == 2) {
+                hipLaunchKernelGGL(chunk_level1_kernel<T>, dim3((unsigned)units), dim3(kWave), 0, stream, path, chunk_low,
+                                   shape, chunks, accumulate ? (T *)nullptr : grad_path);
+            } else {
+                constexpr int PK = P <= N - 2 ? P : N - 2;
+                hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, PK, 1>), dim3((unsigned)units),
+                                   dim3(Geometry<D, N - 1, PK>::kBlock), 0, stream, path, chunk_low, shape, chunks,
+                                   accumulate ? (T *)nullptr : grad_path);
+            }
             e = hipGetLastError();
             if (e != hipSuccess) return e;
         }
@@ -1617,8 +1646,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         }
         int chunks = pick_chunks(rows, v.block, L);
         if (const int64_t forced = options().chunks; forced >= 1 && forced <= 1024) chunks = (int)forced;
-        // not chunked: depth 1 and 2 (the chunked backward needs a level below the top to scan over), units of
-        // several blocks (a row is dozens of waves already), rows too long for the scan kernel's LDS
+        // not chunked: units of several blocks (a row is dozens of waves already), rows too long for the scan
+        // kernel's LDS
         if (!chunks_ok) chunks = 1;
         if (rows * (chunks + 1) >= (int64_t(1) << 31)) return dc;
         dc.usable = true;
