@@ -1298,7 +1298,15 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(119, 49, 2, 1, 1, 1) X(120, 50, 2, 1, 1, 1) X(121, 51, 2, 1, 1, 1) X(122, 52, 2, 1, 1, 1) \
     X(123, 53, 2, 1, 1, 1) X(124, 54, 2, 1, 1, 1) X(125, 55, 2, 1, 1, 1) X(126, 56, 2, 1, 1, 1) \
     X(127, 57, 2, 1, 1, 1) X(128, 58, 2, 1, 1, 1) X(129, 59, 2, 1, 1, 1) X(130, 60, 2, 1, 1, 1) \
-    X(131, 61, 2, 1, 1, 1) X(132, 62, 2, 1, 1, 1) X(133, 63, 2, 1, 1, 1) X(134, 64, 2, 1, 1, 1)
+    X(131, 61, 2, 1, 1, 1) X(132, 62, 2, 1, 1, 1) X(133, 63, 2, 1, 1, 1) X(134, 64, 2, 1, 1, 1) \
+    X(135, 33, 3, 2, 2, 1) X(136, 34, 3, 2, 2, 1) X(137, 35, 3, 2, 2, 1) X(138, 36, 3, 2, 2, 1) \
+    X(139, 37, 3, 2, 2, 1) X(140, 38, 3, 2, 2, 1) X(141, 39, 3, 2, 2, 1) X(142, 40, 3, 2, 2, 1) \
+    X(143, 41, 3, 2, 2, 1) X(144, 42, 3, 2, 2, 1) X(145, 43, 3, 2, 2, 1) X(146, 44, 3, 2, 2, 1) \
+    X(147, 45, 3, 2, 2, 1) X(148, 46, 3, 2, 2, 1) X(149, 47, 3, 2, 2, 1) X(150, 48, 3, 2, 2, 1) \
+    X(151, 49, 3, 2, 2, 1) X(152, 50, 3, 2, 2, 1) X(153, 51, 3, 2, 2, 1) X(154, 52, 3, 2, 2, 1) \
+    X(155, 53, 3, 2, 2, 1) X(156, 54, 3, 2, 2, 1) X(157, 55, 3, 2, 2, 1) X(158, 56, 3, 2, 2, 1) \
+    X(159, 57, 3, 2, 2, 1) X(160, 58, 3, 2, 2, 1) X(161, 59, 3, 2, 2, 1) X(162, 60, 3, 2, 2, 1) \
+    X(163, 61, 3, 2, 2, 1) X(164, 62, 3, 2, 2, 1) X(165, 63, 3, 2, 2, 1) X(166, 64, 3, 2, 2, 1)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.

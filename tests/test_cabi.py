@@ -83,10 +83,10 @@ def test_argument_errors_have_codes_and_messages(lib):
 
 def test_workspace_sizes(lib):
     # general kernels: the forward needs none, the backward one increment accumulator
-    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 33, 3, None, 0) == 0
-    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 33, 3, None, 0)
-    assert need >= 4 * 99 * 33 * 4
-    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 33, 3, None, 0) >= 4 * 99 * 33 * 8
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 65, 3, None, 0) == 0
+    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 65, 3, None, 0)
+    assert need >= 4 * 99 * 65 * 4
+    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 65, 3, None, 0) >= 4 * 99 * 65 * 8
     # a long path on a tiled shape is cut into chunks, which need scratch in the forward too
     assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, None, 0) > 0
     assert lib.pathsig_sig_forward_workspace(0, 4096, 64, 4, 6, None, 0) == 0
@@ -106,7 +106,7 @@ def test_sparse_projections_take_the_dense_kernels_when_that_is_cheaper(lib):
     assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) >= dense
     assert lib.pathsig_sig_forward_workspace(0, 128, 20, 4, 6, sizes(4, 6, 10), 0) == 0      # short path: per word
     assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 6, 6, sizes(6, 6, 10), 0) == 0    # 56 k coefficients: per word
-    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 33, 3, sizes(33, 3, 10), 0) == 0  # no compiled shape
+    assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 65, 3, sizes(65, 3, 10), 0) == 0  # no compiled shape
     try:
         assert lib.pathsig_set_option(b"embed_share", 0) == 0
         assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) == 0

@@ -171,7 +171,7 @@ def test_projection_with_windows(ps, set_option, route):
 @pytest.mark.parametrize("case", [
     dict(d=3, depth=4, L=15, B=13, kind="words"),
     dict(d=3, depth=4, L=40, B=37, kind="gap"),
-    dict(d=33, depth=3, L=23, B=64, kind="dense"),      # no register-tiled shape: all levels dense, per word
+    dict(d=66, depth=3, L=9, B=16, kind="dense"),       # no register-tiled shape: all levels dense, per word
     dict(d=16, depth=6, L=19, B=33, kind="c4"),
     dict(d=2, depth=12, L=9, B=17, kind="long"),
     dict(d=7, depth=5, L=70, B=24, kind="full_low"),
@@ -943,7 +943,7 @@ def test_many_long_rows_fp32_one_chunk(ps, d, depth):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6), (11, 4), (16, 4), (9, 5), (12, 5)])
+@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6), (11, 4), (16, 4), (9, 5), (12, 5), (33, 3), (47, 3), (64, 3)])
 def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
     """d^6 for d >= 6, d^4 for d >= 11, d^5 for d >= 9: a row's lanes (one per prefix) do not fit one block; the
     unit is spread over two to twenty-one blocks, swept in one piece, and the per-increment sums of the backward

@@ -19,7 +19,8 @@ TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (8, 5), (3, 6), (4, 5),
 OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6), (6, 3), (9, 4), (12, 2),
          (11, 4), (20, 3), (3, 8), (2, 10), (27, 2),        # tiled: several blocks per unit, wide, deep
          (45, 2),                                            # tiled, widest kind
-         (70, 2), (2, 11), (35, 3)]                           # no tiled shape: per-word kernels
+         (34, 3),                                            # tiled, several blocks per unit
+         (70, 2), (2, 11), (5, 7)]                            # no tiled shape: per-word kernels
 
 
 def _random_case(rng, ps):
@@ -82,19 +83,23 @@ def test_random_signature_cases(set_option, seed):
         except RuntimeError:  # every window degenerate: the checker's output does not depend on the path
             want_grad = torch.zeros_like(path)
         tol = 1e-5 if dtype == torch.float32 else 1e-12
+        # at depth 10 and more the gradient of a top-level coefficient sums thousands of terms of mixed sign and
+        # fp32 rounding alone passes 1e-5 of the largest gradient: seed 15, case 29 (d = 2, depth 11, windows)
+        # gives 1.04e-5 here and 1.67e-5 in the literal fp32 restatement of the reference's kernel on the CPU
+        tol_grad = 3e-5 if (dtype == torch.float32 and depth >= 10) else tol
         what = f"seed {seed} case {case}: d={d} depth={depth} B={B} L={L} {dtype} windows={windows} chunks={chunks}"
         x = path.to(dtype).to(DEV).requires_grad_(True)
         win = None if windows is None else torch.tensor(windows, dtype=torch.int64, device=DEV)
         mod = ps.Signature(depth=depth, projection=proj, windows=win)
         out = mod(x)
         (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
-        assert rel_err(out, want) < tol and rel_err(grad, want_grad) < tol, what
+        assert rel_err(out, want) < tol and rel_err(grad, want_grad) < tol_grad, what
         args = (mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes, mod.use_windows,
                 mod._windows)
         with torch.no_grad():
             sig = torch.ops.pathsig.compute_signature(x, *args)
             grad = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)
-        assert rel_err(sig, want) < tol and rel_err(grad, want_grad) < tol, what
+        assert rel_err(sig, want) < tol and rel_err(grad, want_grad) < tol_grad, what
         if kind not in ("dense", "lyndon", "aniso") or d ** depth > 5000:
             continue
         # log-signature of the same case; the checker takes the logarithm of the dense signature (by inverting
@@ -113,4 +118,4 @@ def test_random_signature_cases(set_option, seed):
         xl = path.to(dtype).to(DEV).requires_grad_(True)
         lout = ps.LogSignature(depth=depth, projection=proj, windows=win)(xl)
         (lgrad,) = torch.autograd.grad(lout, xl, Gl.to(dtype).to(DEV))
-        assert rel_err(lout, ref.detach()) < tol and rel_err(lgrad, ref_grad) < 5 * tol, "log-signature, " + what
+        assert rel_err(lout, ref.detach()) < tol and rel_err(lgrad, ref_grad) < 5 * tol_grad, "log-signature, " + what
