@@ -403,8 +403,10 @@ struct Geometry {
     // backward then meet in memory).  Such shapes are swept in one piece, without time chunks.
     static constexpr int kUnitWaves = (kLanes + kWave - 1) / kWave;
     // waves of one block: sixteen at most, eight when the lane's sub-trie is large (a block of sixteen waves leaves
-    // each lane 128 registers, which the reverse sweep of such a shape overflows)
-    static constexpr int kMaxWaves = trie_size(D, N - P) > 40 ? 8 : 16;
+    // each lane 128 registers, which the reverse sweep of such a shape overflows); a unit that needs several blocks
+    // anyway takes the smaller block from a smaller sub-trie on
+    static constexpr int kMaxWaves =
+        (trie_size(D, N - P) > 40 || (kUnitWaves > 16 && trie_size(D, N - P) > 30)) ? 8 : 16;
     static constexpr int kWaves = kUnitWaves < kMaxWaves ? kUnitWaves : kMaxWaves;
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
@@ -1306,7 +1308,9 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(151, 49, 3, 2, 2, 1) X(152, 50, 3, 2, 2, 1) X(153, 51, 3, 2, 2, 1) X(154, 52, 3, 2, 2, 1) \
     X(155, 53, 3, 2, 2, 1) X(156, 54, 3, 2, 2, 1) X(157, 55, 3, 2, 2, 1) X(158, 56, 3, 2, 2, 1) \
     X(159, 57, 3, 2, 2, 1) X(160, 58, 3, 2, 2, 1) X(161, 59, 3, 2, 2, 1) X(162, 60, 3, 2, 2, 1) \
-    X(163, 61, 3, 2, 2, 1) X(164, 62, 3, 2, 2, 1) X(165, 63, 3, 2, 2, 1) X(166, 64, 3, 2, 2, 1)
+    X(163, 61, 3, 2, 2, 1) X(164, 62, 3, 2, 2, 1) X(165, 63, 3, 2, 2, 1) X(166, 64, 3, 2, 2, 1) \
+    X(167, 2, 11, 7, 9, 8) X(168, 3, 9, 6, 6, 6) X(169, 3, 10, 7, 6, 6) X(170, 4, 8, 5, 5, 5) \
+    X(171, 5, 7, 5, 5, 4) X(172, 6, 7, 5, 5, 4)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.
@@ -1330,7 +1334,7 @@ template <int D, int N, int P, int PS>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
     return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
-                       LetterBounds<D, P>::kUsable && D <= 16,
+                       LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
                        {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
                         G::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()}};
 }
@@ -1402,7 +1406,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
-    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
     const int64_t rows = shape.B * shape.W;
     if (bounds && !kBoundsOk) return hipErrorInvalidValue;
     if (chunks <= 1) {
@@ -1470,7 +1474,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
                         hipStream_t stream) {
     using G = Geometry<D, N, P>;
     using GC = Geometry<D, N, PS>;
-    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
     const int64_t rows = shape.B * shape.W;
     // per-increment sums are added in memory for overlapping windows and for units spread over several blocks
     const bool accumulate = shape.windows != nullptr || G::kUnitBlocks > 1;

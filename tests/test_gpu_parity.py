@@ -621,7 +621,8 @@ def test_gradcheck(ps):
 TILED = [(4, 6), (8, 4), (6, 5), (4, 4), (3, 5), (2, 8), (3, 6), (4, 5), (5, 4), (5, 5), (5, 6), (6, 4), (7, 4), (7, 5),
          (2, 2), (5, 2), (8, 2), (2, 3), (3, 3), (6, 3), (7, 3), (8, 3), (2, 4), (3, 4), (2, 5), (2, 6),
          (9, 2), (13, 2), (16, 2), (9, 3), (11, 3), (16, 3), (9, 4), (10, 4), (2, 7), (3, 7), (4, 7), (3, 8), (2, 9), (2, 10),
-         (17, 2), (32, 2), (17, 3), (27, 3), (32, 3), (33, 2), (50, 2), (64, 2)]
+         (17, 2), (32, 2), (17, 3), (27, 3), (32, 3), (33, 2), (50, 2), (64, 2),
+         (2, 11), (3, 9)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -943,7 +944,8 @@ def test_many_long_rows_fp32_one_chunk(ps, d, depth):
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
-@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6), (11, 4), (16, 4), (9, 5), (12, 5), (33, 3), (47, 3), (64, 3)])
+@pytest.mark.parametrize("d,depth", [(6, 6), (7, 6), (8, 6), (11, 4), (16, 4), (9, 5), (12, 5), (33, 3), (47, 3), (64, 3),
+                                     (3, 10), (4, 8), (5, 7), (6, 7)])
 def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
     """d^6 for d >= 6, d^4 for d >= 11, d^5 for d >= 9: a row's lanes (one per prefix) do not fit one block; the
     unit is spread over two to twenty-one blocks, swept in one piece, and the per-increment sums of the backward

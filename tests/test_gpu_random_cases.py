@@ -20,7 +20,8 @@ OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6)
          (11, 4), (20, 3), (3, 8), (2, 10), (27, 2),        # tiled: several blocks per unit, wide, deep
          (45, 2),                                            # tiled, widest kind
          (34, 3),                                            # tiled, several blocks per unit
-         (70, 2), (2, 11), (5, 7)]                            # no tiled shape: per-word kernels
+         (2, 11),                                            # tiled, deep
+         (70, 2), (100, 2)]                                  # no tiled shape: per-word kernels
 
 
 def _random_case(rng, ps):
