@@ -6,8 +6,9 @@
 // every lane that shares them) and the whole sub-trie below u (levels P+1..N, sum_k D^k values) in
 // registers.  All letters below u are compile-time constants, so every state access is a fixed
 // register and the increment of the step is the same for all lanes of the unit: there is no
-// inter-lane traffic and no barrier inside the time loop.  One "unit" = one (path, window); its D^P
-// lanes fill ceil(D^P / 64) wavefronts of one workgroup, which stages a tile of increments in LDS.
+// inter-lane traffic and no barrier inside the time loop.  One "unit" = one (path, window, time chunk); its
+// D^P lanes fill ceil(D^P / 64) wavefronts of one workgroup (of several for the largest shapes), each of
+// which stages a tile of increments in LDS.
 //
 // Horner form of one step for target level m (every node is one FMA):
 //     tmp_j[w a] = S_j[w a] + (tmp_{j-1}[w] / (m - j + 1)) * dx[a],   j = 1..m-1,   tmp_0 = 1
