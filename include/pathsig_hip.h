@@ -173,6 +173,7 @@ int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const vo
  *                     wanted columns) instead of the per-word kernels: -1 = the library's rule (top level keeps
  *                     1/8 of the dense one, or the dense sweep is estimated cheaper), 0 = none, n > 0 = those whose
  *                     top level keeps at least 1/n of the dense one (PATHSIG_EMBED_SHARE)
+ *   "tiled"           0 = every call takes the per-word kernels, whatever its shape (PATHSIG_NO_TILED sets 0)
  * Returns PATHSIG_ERR_ARGUMENT for an unknown name or a value out of range.
  */
 int pathsig_set_option(const char *name, int64_t value);

@@ -37,13 +37,14 @@ int64_t env_int(const char *name, int64_t fallback) {
 
 // Plain integers behind relaxed atomics: a setter on one thread and a call on another see whole values.
 struct OptionCells {
-    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share;
+    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share, tiled;
     OptionCells()
         : chunks(env_int("PATHSIG_CHUNKS", 0)),
           letter_bounds(getenv("PATHSIG_NO_LETTER_BOUNDS") ? 0 : 1),
           logsig_scatter(env_int("PATHSIG_LOGSIG_SCATTER", 0) == 1 ? 1 : 0),
           batch_tile(env_int("PATHSIG_BATCH_TILE", 0)),
-          embed_share(env_int("PATHSIG_EMBED_SHARE", -1)) {}
+          embed_share(env_int("PATHSIG_EMBED_SHARE", -1)),
+          tiled(getenv("PATHSIG_NO_TILED") ? 0 : 1) {}
 };
 OptionCells &option_cells() {
     static OptionCells cells;  // the environment is read here, once
@@ -59,6 +60,7 @@ const Options &options() {
     snapshot.logsig_scatter = c.logsig_scatter.load(std::memory_order_relaxed);
     snapshot.batch_tile = c.batch_tile.load(std::memory_order_relaxed);
     snapshot.embed_share = c.embed_share.load(std::memory_order_relaxed);
+    snapshot.tiled = c.tiled.load(std::memory_order_relaxed);
     return snapshot;
 }
 
@@ -367,6 +369,8 @@ int pathsig_set_option(const char *name, int64_t value) {
         option_cells().batch_tile.store(value, std::memory_order_relaxed);
     } else if (!strcmp(name, "embed_share") && value >= -1) {
         option_cells().embed_share.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "tiled") && (value == 0 || value == 1)) {
+        option_cells().tiled.store(value, std::memory_order_relaxed);
     } else {
         set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
         return PATHSIG_ERR_ARGUMENT;

@@ -50,6 +50,7 @@ struct Options {
     int64_t batch_tile;      // cap on the increments per tile of the lanes-on-paths backward (0: no cap)
     int64_t embed_share;     // a projection runs on the register-tiled kernels when its top level keeps at least
                              // 1/embed_share of the dense one (0: never; -1: the library's own rule)
+    int64_t tiled;           // 0: every call takes the per-word kernels, whatever its shape (default 1)
 };
 const Options &options();
 

@@ -1610,7 +1610,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
     DenseChoice dc{};
     dc.variant = -1;
     dc.fwd_chunks = dc.bwd_chunks = 1;
-    if (B <= 0 || W <= 0) return dc;
+    if (B <= 0 || W <= 0 || options().tiled == 0) return dc;
     for (int i = 0; i < kNumVariants; ++i) {
         const VariantInfo &v = kVariants[i];
         if (v.d != d || v.depth != depth) continue;

@@ -112,5 +112,9 @@ def test_sparse_projections_take_the_dense_kernels_when_that_is_cheaper(lib):
         assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) == 0
         assert lib.pathsig_set_option(b"embed_share", 10 ** 9) == 0
         assert lib.pathsig_sig_forward_workspace(0, 128, 20, 4, 6, sizes(4, 6, 10), 0) >= dense
+        assert lib.pathsig_set_option(b"tiled", 0) == 0                  # no tiled kernels at all: no dense buffer
+        assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, sizes(4, 6, 10), 0) == 0
+        assert lib.pathsig_set_option(b"tiled", 2) != 0
     finally:
         assert lib.pathsig_set_option(b"embed_share", -1) == 0
+        assert lib.pathsig_set_option(b"tiled", 1) == 0

@@ -958,3 +958,24 @@ def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
         got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
         assert rel_err(got, want) < TOL[dtype]
         assert rel_err(grad, TO.signature_vjp(path, G, depth, None, None, windows)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,B", [(4, 6, 2), (8, 4, 3), (2, 8, 70), (16, 3, 5), (3, 5, 130), (20, 2, 9)])
+def test_per_word_kernels_on_shapes_that_have_a_tiled_kernel(ps, set_option, dtype, d, depth, B):
+    """With the tiled kernels switched off the same dense calls run on the per-word kernels (lanes on words for few
+    paths, lanes on paths for many): both families must agree with the checker, and with each other to rounding."""
+    L = 12
+    path = brownian_path(B, L, d, seed=900 + d)
+    for windows in (None, [(0, 12), (3, 9), (4, 5), (7, 7)]):
+        want = TO.compute_signature(path, depth, None, None, windows)
+        G = randn(tuple(want.shape), seed=901)
+        want_grad = TO.signature_vjp(path, G, depth, None, None, windows)
+        results = []
+        for tiled in (0, 1):
+            set_option("tiled", tiled)
+            got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
+            assert rel_err(got, want) < TOL[dtype] and rel_err(grad, want_grad) < TOL[dtype], f"tiled={tiled}"
+            results.append((got, grad))
+        assert rel_err(results[0][0], results[1][0]) < TOL[dtype]
+        assert rel_err(results[0][1], results[1][1]) < TOL[dtype]
