@@ -20,7 +20,7 @@ OTHER = [(2, 3), (3, 4), (5, 3), (7, 2), (2, 7), (3, 7), (16, 3), (9, 3), (2, 6)
          (11, 4), (20, 3), (3, 8), (2, 10), (27, 2),        # tiled: several blocks per unit, wide, deep
          (45, 2),                                            # tiled, widest kind
          (34, 3),                                            # tiled, several blocks per unit
-         (2, 11),                                            # tiled, deep
+         (2, 11), (2, 12),                                   # tiled, deep
          (70, 2), (100, 2)]                                  # no tiled shape: per-word kernels
 
 
