@@ -407,7 +407,8 @@ struct Geometry {
     // each lane 128 registers, which the reverse sweep of such a shape overflows); a unit that needs several blocks
     // anyway takes the smaller block from a smaller sub-trie on
     static constexpr int kMaxWaves =
-        (trie_size(D, N - P) > 40 || (kUnitWaves > 16 && trie_size(D, N - P) > 30)) ? 8 : 16;
+        trie_size(D, N - P) > 160 ? 4
+        : (trie_size(D, N - P) > 40 || (kUnitWaves > 16 && trie_size(D, N - P) > 30)) ? 8 : 16;
     static constexpr int kWaves = kUnitWaves < kMaxWaves ? kUnitWaves : kMaxWaves;
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
@@ -1281,10 +1282,10 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(39, 11, 2, 1, 1, 1) X(40, 12, 2, 1, 1, 1) X(41, 13, 2, 1, 1, 1) X(42, 14, 2, 1, 1, 1) \
     X(43, 15, 2, 1, 1, 1) X(44, 16, 2, 1, 1, 1) X(45, 9, 3, 2, 2, 1) X(46, 10, 3, 2, 2, 1) \
     X(47, 11, 3, 2, 2, 1) X(48, 12, 3, 2, 2, 1) X(49, 13, 3, 2, 2, 1) X(50, 14, 3, 2, 2, 1) \
-    X(51, 15, 3, 2, 2, 1) X(52, 16, 3, 2, 2, 1) X(53, 9, 4, 3, 3, 2) X(54, 10, 4, 3, 3, 2) \
-    X(55, 11, 4, 3, 3, 2) X(56, 12, 4, 3, 3, 2) X(57, 13, 4, 3, 3, 2) X(58, 14, 4, 3, 3, 2) \
-    X(59, 15, 4, 3, 3, 2) X(60, 16, 4, 3, 3, 2) X(61, 9, 5, 4, 4, 3) X(62, 10, 5, 4, 4, 3) \
-    X(63, 11, 5, 4, 4, 3) X(64, 12, 5, 4, 4, 3) X(65, 2, 7, 5, 6, 5) X(66, 3, 7, 4, 5, 4) \
+    X(51, 15, 3, 2, 2, 1) X(52, 16, 3, 2, 2, 1) X(53, 9, 4, 2, 3, 2) X(54, 10, 4, 2, 3, 2) \
+    X(55, 11, 4, 2, 3, 2) X(56, 12, 4, 2, 3, 2) X(57, 13, 4, 2, 3, 2) X(58, 14, 4, 2, 3, 2) \
+    X(59, 15, 4, 2, 3, 2) X(60, 16, 4, 3, 3, 2) X(61, 9, 5, 3, 3, 3) X(62, 10, 5, 3, 3, 3) \
+    X(63, 11, 5, 3, 3, 3) X(64, 12, 5, 3, 3, 3) X(65, 2, 7, 5, 6, 5) X(66, 3, 7, 4, 5, 4) \
     X(67, 4, 7, 4, 5, 4) X(68, 3, 8, 5, 6, 5) X(69, 2, 9, 6, 8, 7) X(70, 2, 10, 6, 8, 7) \
     X(71, 17, 2, 1, 1, 1) X(72, 18, 2, 1, 1, 1) X(73, 19, 2, 1, 1, 1) X(74, 20, 2, 1, 1, 1) \
     X(75, 21, 2, 1, 1, 1) X(76, 22, 2, 1, 1, 1) X(77, 23, 2, 1, 1, 1) X(78, 24, 2, 1, 1, 1) \
@@ -1314,13 +1315,18 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     X(171, 5, 7, 5, 5, 4) X(172, 6, 7, 5, 5, 4) X(173, 2, 12, 7, 9, 8) X(174, 7, 7, 5, 5, 4) \
     X(175, 8, 7, 5, 5, 4) X(176, 4, 9, 6, 6, 6) X(177, 3, 11, 8, 6, 6) \
     X(178, 3, 12, 9, 6, 6) X(179, 4, 10, 7, 6, 6) X(180, 4, 11, 8, 6, 6) X(181, 5, 8, 6, 5, 5) \
-    X(182, 5, 9, 7, 5, 5) X(183, 6, 8, 6, 5, 5) X(184, 7, 8, 6, 5, 5) X(185, 9, 6, 5, 5, 4) \
-    X(186, 10, 6, 5, 5, 4) X(187, 11, 6, 5, 5, 4) X(188, 12, 6, 5, 5, 4) X(189, 13, 5, 4, 4, 3) \
-    X(190, 14, 5, 4, 4, 3) X(191, 15, 5, 4, 4, 3) X(192, 16, 5, 4, 4, 3) X(193, 17, 4, 3, 3, 2) \
+    X(182, 5, 9, 7, 5, 5) X(183, 6, 8, 6, 5, 5) X(184, 7, 8, 6, 5, 5) X(185, 9, 6, 4, 4, 3) \
+    X(186, 10, 6, 4, 4, 3) X(187, 11, 6, 4, 4, 3) X(188, 12, 6, 4, 4, 3) X(189, 13, 5, 3, 3, 3) \
+    X(190, 14, 5, 3, 3, 3) X(191, 15, 5, 3, 3, 3) X(192, 16, 5, 4, 4, 3) X(193, 17, 4, 3, 3, 2) \
     X(194, 18, 4, 3, 3, 2) X(195, 19, 4, 3, 3, 2) X(196, 20, 4, 3, 3, 2) X(197, 21, 4, 3, 3, 2) \
     X(198, 22, 4, 3, 3, 2) X(199, 23, 4, 3, 3, 2) X(200, 24, 4, 3, 3, 2) X(201, 25, 4, 3, 3, 2) \
     X(202, 26, 4, 3, 3, 2) X(203, 27, 4, 3, 3, 2) X(204, 28, 4, 3, 3, 2) X(205, 29, 4, 3, 3, 2) \
-    X(206, 30, 4, 3, 3, 2) X(207, 31, 4, 3, 3, 2) X(208, 32, 4, 3, 3, 2)
+    X(206, 30, 4, 3, 3, 2) X(207, 31, 4, 3, 3, 2) X(208, 32, 4, 3, 3, 2) \
+    X(209, 9, 4, 3, 3, 2) X(210, 10, 4, 3, 3, 2) X(211, 11, 4, 3, 3, 2) X(212, 12, 4, 3, 3, 2) \
+    X(213, 13, 4, 3, 3, 2) X(214, 14, 4, 3, 3, 2) X(215, 15, 4, 3, 3, 2) X(216, 9, 5, 4, 4, 3) \
+    X(217, 10, 5, 4, 4, 3) X(218, 11, 5, 4, 4, 3) X(219, 12, 5, 4, 4, 3) X(220, 13, 5, 4, 4, 3) \
+    X(221, 14, 5, 4, 4, 3) X(222, 15, 5, 4, 4, 3) X(223, 9, 6, 5, 5, 4) X(224, 10, 6, 5, 5, 4) \
+    X(225, 11, 6, 5, 5, 4) X(226, 12, 6, 5, 5, 4)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.
@@ -1338,6 +1344,7 @@ struct VariantInfo {
     int64_t sig_size, low_size;
     bool bounds_ok;       // the sweeps can leave out top-level words by letter bounds
     bool chunks_ok[2];    // fp32, fp64: rows can be cut into time chunks
+    bool fp64_fits;       // a lane's state fits the register file in fp64 too (else a later entry of the shape serves fp64)
 };
 
 template <int D, int N, int P, int PS>
@@ -1346,7 +1353,8 @@ constexpr VariantInfo variant_info() {
     return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
                        LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
                        {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
-                        G::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()}};
+                        G::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
+                       trie_size(D, N - P) <= 88};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1631,6 +1639,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             for (int j = i + 1; j < kNumVariants; ++j) later = later || (kVariants[j].d == d && kVariants[j].depth == depth);
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
+            // the short prefixes of the wide alphabets hold 90 to 240 values per lane: fp32 only
+            if (later && elem == 8 && !v.fp64_fits) continue;
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
         if (!all_dense) {

@@ -1001,3 +1001,22 @@ def test_per_word_kernels_on_shapes_that_have_a_tiled_kernel(ps, set_option, dty
             results.append((got, grad))
         assert rel_err(results[0][0], results[1][0]) < TOL[dtype]
         assert rel_err(results[0][1], results[1][1]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,B,L", [(9, 4, 64, 150), (12, 4, 64, 150), (13, 4, 64, 150), (15, 4, 64, 150),
+                                         (9, 5, 12, 150), (12, 5, 12, 150), (13, 5, 12, 150), (15, 5, 12, 40),
+                                         (9, 6, 6, 40), (12, 6, 2, 24)])
+def test_wide_alphabets_with_enough_rows_for_the_short_prefix(ps, dtype, d, depth, B, L):
+    """d = 9..15 at depth 4 and 5 and d = 9..12 at depth 6 are compiled twice: lanes on prefixes of length depth - 2 (90 to 240 values per lane,
+    fp32 only, taken when the rows fill the device) and of length depth - 1 (fp64, few rows).  Enough rows here for
+    the first kind; the checker runs on two of them."""
+    path = brownian_path(B, L, d, seed=800 + d + depth)
+    x = path.to(dtype).to(DEV).requires_grad_(True)
+    out = ps.Signature(depth=depth)(x)
+    G = randn(tuple(out.shape), seed=801)
+    (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+    idx = torch.tensor([0, B - 1])
+    want = TO.signature(path[idx], depth)
+    assert rel_err(out.detach().cpu()[idx], want) < TOL[dtype]
+    assert rel_err(grad.cpu()[idx], TO.signature_vjp(path[idx], G[idx], depth)) < TOL[dtype]
