@@ -396,7 +396,7 @@ __device__ __forceinline__ void read_increments(const T *sdx, int tt, const int 
 
 constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2) : 1; }
 
-template <int D, int N, int P>
+template <int D, int N, int P, int ELEM = 4>
 struct Geometry {
     static constexpr int kLanes = ipow(D, P);
     // A unit needs kUnitWaves waves.  Up to sixteen of them form one block; a larger unit is spread over
@@ -404,11 +404,21 @@ struct Geometry {
     // backward then meet in memory).  Such shapes are swept in one piece, without time chunks.
     static constexpr int kUnitWaves = (kLanes + kWave - 1) / kWave;
     // waves of one block: sixteen at most, eight when the lane's sub-trie is large (a block of sixteen waves leaves
-    // each lane 128 registers, which the reverse sweep of such a shape overflows); a unit that needs several blocks
+    // each lane 128 registers, which the reverse sweep of such a shape overflows), four from 160 values on (one
+    // wave per SIMD: 512 registers, the upper half reached through copies); a unit that needs several blocks
     // anyway takes the smaller block from a smaller sub-trie on
+    static constexpr int kSubTrie = trie_size(D, N - P);
+    static constexpr int kMaxWaves32 =
+        kSubTrie > 160 ? 4 : (kSubTrie > 40 || (kUnitWaves > 16 && kSubTrie > 30)) ? 8 : 16;
+    // fp64 doubles the registers of a lane's state.  Where the unit is spread over several blocks anyway (or,
+    // with three levels below the prefix, would fill more than eight waves), the blocks shrink until the state
+    // fits: the reverse sweeps of these shapes spilled 200 to 400 registers to memory in blocks of eight or
+    // sixteen waves.  Units of one block keep their shape (they may be cut into time chunks).
+    static constexpr bool kSplit64 = ELEM == 8 && (kUnitWaves > kMaxWaves32 || (N - P >= 3 && kUnitWaves > 8));
     static constexpr int kMaxWaves =
-        trie_size(D, N - P) > 160 ? 4
-        : (trie_size(D, N - P) > 40 || (kUnitWaves > 16 && trie_size(D, N - P) > 30)) ? 8 : 16;
+        !kSplit64 ? kMaxWaves32
+        : (kSubTrie >= 72 || N - P >= 3 || (kSubTrie >= 56 && P >= 6)) ? 4
+        : kSubTrie >= 30 ? (kMaxWaves32 < 8 ? kMaxWaves32 : 8) : kMaxWaves32;
     static constexpr int kWaves = kUnitWaves < kMaxWaves ? kUnitWaves : kMaxWaves;
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
@@ -594,14 +604,14 @@ __device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], 
 // ---------------------------------------------------------------------------------------------
 template <int D, int N, int P, int GW, typename T>
 constexpr size_t forward_lds_bytes() {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     return (size_t)GW * kTile * (N - P) * D * sizeof(T) + (size_t)(GW / 2) * G::kSigSize * sizeof(T);
 }
 
 // LDS layout of the forward sweep: staged increments per chunk, and slots for the in-block products
 template <typename T, int D, int N, int P, int GW>
 struct ForwardShape {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     static constexpr int KS = N - P;
     static constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
     static constexpr int kSlotSize = GW > 1 ? (int)G::kSigSize : 4;
@@ -622,7 +632,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
                                                    T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW>::kStage],
                                                    T (&slot)[ForwardShape<T, D, N, P, GW>::kSlots]
                                                             [ForwardShape<T, D, N, P, GW>::kSlotSize]) {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     constexpr int KS = N - P;
     const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
     T *sdx = sdx_all[part];
@@ -708,7 +718,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
 // the copy of the sweep compiled for its bound; the copies differ in nothing but the sub-trie nodes they leave
 // out, so all waves of the block still meet at the same barriers.
 template <typename T, int D, int N, int P, int GW, bool BOUNDED = false>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
+__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
                          T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr,
                          T *__restrict__ chunk_low = nullptr) {
@@ -716,7 +726,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock * GW))
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
     __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     static_assert(G::kUnitBlocks == 1 || (GW == 1 && !BOUNDED), "a unit of several blocks is swept one chunk to a block");
     const int tid = (int)threadIdx.x % G::kBlock;
     if constexpr (BOUNDED) {
@@ -1013,7 +1023,7 @@ __global__ void __launch_bounds__(kWave) chunk_level1_kernel(const T *__restrict
 // widest alphabets, whose parts of sixteen increments would not fit a CU at all).
 template <typename T, int D, int N, int P>
 struct BackwardShape {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     static constexpr int KS = N - P;
     static constexpr int kParts = 4;
     static constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
@@ -1042,7 +1052,7 @@ __device__ __forceinline__ void dense_backward_body(
     T (&sdx)[BackwardShape<T, D, N, P>::kStage],
     T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
     T (&cells)[BackwardShape<T, D, N, P>::kCells]) {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     using BS = BackwardShape<T, D, N, P>;
     constexpr int KS = N - P;
     constexpr int kParts = BS::kParts;
@@ -1232,7 +1242,7 @@ __device__ __forceinline__ void dense_backward_body(
 // LetterBounds).  Every wave runs the copy of the sweep compiled for its bound; all copies meet at the same
 // barriers.
 template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, bool BOUNDED = false>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
                           const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
                           SigShape shape, int chunks, T *__restrict__ grad_path = nullptr,
@@ -1242,7 +1252,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
     __shared__ __align__(16) T sdx[BS::kStage];
     __shared__ T sg[BS::kSums][BS::kSumRow];
     __shared__ T cells[BS::kCells];
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     static_assert(G::kUnitBlocks == 1 || (ACCUMULATE && !CHUNKED && !BOUNDED),
                   "a unit of several blocks is swept in one piece and adds its per-increment sums in memory");
     const int tid = (int)threadIdx.x;
@@ -1350,10 +1360,11 @@ struct VariantInfo {
 template <int D, int N, int P, int PS>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
+    using G64 = Geometry<D, N, P, 8>;
     return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
                        LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
                        {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
-                        G::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
+                        G64::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
                        trie_size(D, N - P) <= 88};
 }
 
@@ -1415,13 +1426,13 @@ int pick_chunks(int64_t rows, int block, int64_t L) {
 
 template <typename T, int D, int N, int P, int GW>
 constexpr bool group_fits() {
-    return Geometry<D, N, P>::kBlock * GW <= 1024 && forward_lds_bytes<D, N, P, GW, T>() <= 64 * 1024;
+    return Geometry<D, N, P, sizeof(T)>::kBlock * GW <= 1024 && forward_lds_bytes<D, N, P, GW, T>() <= 64 * 1024;
 }
 
 template <typename T, int D, int N, int P, int PC>
 hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, T *keep,
                        void *workspace, hipStream_t stream) {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
@@ -1490,7 +1501,7 @@ template <typename T, int D, int N, int P, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
                         const SigShape &shape, int chunks, const int *bounds, const T *kept, void *workspace,
                         hipStream_t stream) {
-    using G = Geometry<D, N, P>;
+    using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PS>;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
     const int64_t rows = shape.B * shape.W;
@@ -1545,7 +1556,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             } else {
                 constexpr int PK = P <= N - 2 ? P : N - 2;
                 hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, PK, 1>), dim3((unsigned)units),
-                                   dim3(Geometry<D, N - 1, PK>::kBlock), 0, stream, path, chunk_low, shape, chunks,
+                                   dim3(Geometry<D, N - 1, PK, sizeof(T)>::kBlock), 0, stream, path, chunk_low, shape, chunks,
                                    accumulate ? (T *)nullptr : grad_path);
             }
             e = hipGetLastError();
