@@ -1365,7 +1365,7 @@ constexpr VariantInfo variant_info() {
                        LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
                        {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
                         G64::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
-                       trie_size(D, N - P) <= 88};
+                       trie_size(D, N - P) <= 132};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1650,7 +1650,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             for (int j = i + 1; j < kNumVariants; ++j) later = later || (kVariants[j].d == d && kVariants[j].depth == depth);
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
-            // the short prefixes of the wide alphabets hold 90 to 240 values per lane: fp32 only
+            // the short prefixes of the wide alphabets hold 90 to 240 values per lane: fp64 up to 132 (d = 11)
             if (later && elem == 8 && !v.fp64_fits) continue;
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
