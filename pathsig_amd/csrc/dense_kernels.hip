@@ -62,6 +62,30 @@ __device__ __forceinline__ void dispatch_value(int value, F &&f) {
 constexpr int ipow(int b, int e) { return e <= 0 ? 1 : b * ipow(b, e - 1); }
 // number of sub-trie values in levels 1..k below a prefix
 constexpr int trie_size(int D, int k) { return k <= 0 ? 0 : ipow(D, k) + trie_size(D, k - 1); }
+// values on the first k levels below a lane's prefix when the lane holds K children of the prefix (all D of them
+// unless the first level is split between several lanes) and every child's complete sub-trie
+constexpr int sub_size(int D, int K, int k) { return k <= 0 ? 0 : K * ipow(D, k - 1) + sub_size(D, K, k - 1); }
+// Children of the prefix that one lane holds.  The widest alphabets at depth 4 and 5 split them between lanes: with
+// all D children a lane would hold D + D^2 = 272 values and more, with the next longer prefix only D.
+// Chosen by an estimate of the useful share of a lane's instructions: K / (K + 1.5) for the chain, the per-letter
+// sums and the reduction that every lane pays whatever K is, times the share of child slots in use (the last lane
+// of a prefix may hold fewer than K), within K * (D + 1) <= 136 values.
+constexpr int split_children(int D, int N, int P) {
+    if (!(D >= 16 && D <= 32 && P == N - 2 && (N == 4 || (N == 5 && D == 16)))) return D;
+    int best = 2;
+    long best_num = 0, best_den = 1;
+    for (int k = 2; k * (D + 1) <= 136 && k <= 8; ++k) {
+        const int parts = (D + k - 1) / k;
+        // D / (parts * k) * k / (k + 1.5)  =  2 D / (parts * (2 k + 3))
+        const long num = 2L * D, den = (long)parts * (2 * k + 3);
+        if (num * best_den >= best_num * den) {
+            best = k;
+            best_num = num;
+            best_den = den;
+        }
+    }
+    return best;
+}
 
 template <typename T>
 __device__ __forceinline__ constexpr T rcp(int k) { return T(1) / T(k); }
@@ -81,31 +105,37 @@ __device__ __forceinline__ double fmad<double>(double a, double b, double c) { r
 // On the chain (P nodes per target) the parent is scaled instead.
 // ---------------------------------------------------------------------------------------------
 // LO: letters below LO are left out below the prefix (their words are not wanted; see LetterBounds).
-template <typename T, int D, int P, int M, int J, bool NEG, int LO = 0>
+// K: children of the prefix held by the lane (D, or fewer when the first level is split between lanes: then dxf
+// holds the scaled increments of the lane's own K letters; otherwise dxf is dxs).
+template <typename T, int D, int P, int M, int J, bool NEG, int LO = 0, int K = D>
 struct StepDescend {
     // children (level J > P) of a node with Horner value pt; idx0 = index of the first child within level J
     template <int SUB, int KS>
-    static __device__ __forceinline__ void run(T pt, int idx0, T (&sub)[SUB], const T (&dxs)[KS][D]) {
-        constexpr int off = trie_size(D, J - P - 1);
+    static __device__ __forceinline__ void run(T pt, int idx0, T (&sub)[SUB], const T (&dxs)[KS][D],
+                                               const T (&dxf)[KS][K]) {
+        constexpr int off = sub_size(D, K, J - P - 1);
+        constexpr bool kFirst = J == P + 1;
 #pragma unroll
-        for (int a = LO; a < D; ++a) {
-            const T inc = NEG ? -dxs[M - J][a] : dxs[M - J][a];
+        for (int a = LO; a < (kFirst ? K : D); ++a) {
+            T inc;
+            if constexpr (kFirst) inc = NEG ? -dxf[M - J][a] : dxf[M - J][a];
+            else inc = NEG ? -dxs[M - J][a] : dxs[M - J][a];
             if constexpr (J == M) {
                 sub[off + idx0 + a] = fmad<T>(pt, inc, sub[off + idx0 + a]);
             } else {
                 const T tmp = fmad<T>(pt, inc, sub[off + idx0 + a]);
-                StepDescend<T, D, P, M, J + 1, NEG, LO>::template run<SUB, KS>(tmp, (idx0 + a) * D, sub, dxs);
+                StepDescend<T, D, P, M, J + 1, NEG, LO, K>::template run<SUB, KS>(tmp, (idx0 + a) * D, sub, dxs, dxf);
             }
         }
     }
 };
 
 // LO applies to the top target only (the first M of the recursion); the targets below are complete.
-template <typename T, int D, int P, int M, bool NEG, int LO = 0>
+template <typename T, int D, int P, int M, bool NEG, int LO = 0, int K = D>
 struct StepTargets {
     template <int SUB, int KS>
     static __device__ __forceinline__ void run(T (&a)[P + 1], T (&sub)[SUB], const T (&dxs)[KS][D],
-                                               const T (&dxp)[P]) {
+                                               const T (&dxf)[KS][K], const T (&dxp)[P]) {
         T ps = rcp<T>(M);
         T tmp = T(1);
         constexpr int JP = (M - 1 < P) ? (M - 1) : P;
@@ -117,50 +147,59 @@ struct StepTargets {
         if constexpr (M <= P) {
             a[M] = fmad<T>(ps, NEG ? -dxp[M - 1] : dxp[M - 1], a[M]);
         } else {
-            StepDescend<T, D, P, M, P + 1, NEG, LO>::template run<SUB, KS>(tmp, 0, sub, dxs);
+            StepDescend<T, D, P, M, P + 1, NEG, LO, K>::template run<SUB, KS>(tmp, 0, sub, dxs, dxf);
         }
-        if constexpr (M > 1) StepTargets<T, D, P, M - 1, NEG>::template run<SUB, KS>(a, sub, dxs, dxp);
+        if constexpr (M > 1) StepTargets<T, D, P, M - 1, NEG, 0, K>::template run<SUB, KS>(a, sub, dxs, dxf, dxp);
     }
 };
 
 // ---------------------------------------------------------------------------------------------
 // adjoint of one Chen step
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int P, int M, int J, int LO = 0>
+template <typename T, int D, int P, int M, int J, int LO = 0, int K = D>
 struct AdjDescend {
     // pt = Horner value of the parent; returns its adjoint.  gdxk[q][a] collects the gradient with respect
     // to dxs[q][a]; the caller folds the 1/(q+1) back in.
     template <int ASUB, int HSUB, int KS>
+    // (with the first level split between lanes: dxf / gdxf are the increments of the lane's own K letters and
+    // their gradients; otherwise they are dxs / gdxk themselves)
     static __device__ __forceinline__ T run(T pt, int idx0, const T (&asub)[ASUB], T (&hsub)[HSUB],
-                                            const T (&dxs)[KS][D], T (&gdxk)[KS][D]) {
-        constexpr int off = trie_size(D, J - P - 1);
+                                            const T (&dxs)[KS][D], const T (&dxf)[KS][K], T (&gdxk)[KS][D],
+                                            T (&gdxf)[KS][K]) {
+        constexpr int off = sub_size(D, K, J - P - 1);
+        constexpr bool kFirst = J == P + 1;
         T gpt = T(0);
 #pragma unroll
-        for (int a = LO; a < D; ++a) {
+        for (int a = LO; a < (kFirst ? K : D); ++a) {
+            T inc;
+            if constexpr (kFirst) inc = dxf[M - J][a];
+            else inc = dxs[M - J][a];
             T g;
             if constexpr (J == M) {
                 g = hsub[off + idx0 + a];
             } else {
-                const T tmp = fmad<T>(pt, dxs[M - J][a], asub[off + idx0 + a]);
-                g = AdjDescend<T, D, P, M, J + 1, LO>::template run<ASUB, HSUB, KS>(tmp, (idx0 + a) * D, asub, hsub,
-                                                                                    dxs, gdxk);
+                const T tmp = fmad<T>(pt, inc, asub[off + idx0 + a]);
+                g = AdjDescend<T, D, P, M, J + 1, LO, K>::template run<ASUB, HSUB, KS>(tmp, (idx0 + a) * D, asub, hsub,
+                                                                                       dxs, dxf, gdxk, gdxf);
                 hsub[off + idx0 + a] += g;
             }
-            gdxk[M - J][a] = fmad<T>(g, pt, gdxk[M - J][a]);
-            gpt = fmad<T>(g, dxs[M - J][a], gpt);
+            if constexpr (kFirst) gdxf[M - J][a] = fmad<T>(g, pt, gdxf[M - J][a]);
+            else gdxk[M - J][a] = fmad<T>(g, pt, gdxk[M - J][a]);
+            gpt = fmad<T>(g, inc, gpt);
         }
         return gpt;
     }
 };
 
-template <typename T, int D, int N, int P, int M, int LO = 0>
+template <typename T, int D, int N, int P, int M, int LO = 0, int K = D>
 struct AdjTargets {
     // targets ascending: the seed of target M (adjoint of level M) is only changed by targets above M;
     // LO applies to the top target (M = N), whose left-out words have a zero upstream gradient
     template <int ASUB, int HSUB, int KS>
     static __device__ __forceinline__ void run(const T (&a)[P + 1], const T (&asub)[ASUB], T (&hc)[P + 1],
-                                               T (&hsub)[HSUB], const T (&dxs)[KS][D], const T (&dxp)[P],
-                                               T (&gdxk)[KS][D], T (&gpre)[P]) {
+                                               T (&hsub)[HSUB], const T (&dxs)[KS][D], const T (&dxf)[KS][K],
+                                               const T (&dxp)[P], T (&gdxk)[KS][D], T (&gdxf)[KS][K],
+                                               T (&gpre)[P]) {
         constexpr int JP = (M - 1 < P) ? (M - 1) : P;
         T ps[P + 2];
         T tmp = T(1);
@@ -175,8 +214,8 @@ struct AdjTargets {
         if constexpr (M <= P) {
             g = hc[M];
         } else {
-            g = AdjDescend<T, D, P, M, P + 1, (M == N ? LO : 0)>::template run<ASUB, HSUB, KS>(tmp, 0, asub, hsub, dxs,
-                                                                                                 gdxk);
+            g = AdjDescend<T, D, P, M, P + 1, (M == N ? LO : 0), K>::template run<ASUB, HSUB, KS>(
+                tmp, 0, asub, hsub, dxs, dxf, gdxk, gdxf);
             hc[P] += g;
         }
 #pragma unroll
@@ -188,7 +227,8 @@ struct AdjTargets {
             }
         }
         if constexpr (M < N)
-            AdjTargets<T, D, N, P, M + 1, LO>::template run<ASUB, HSUB, KS>(a, asub, hc, hsub, dxs, dxp, gdxk, gpre);
+            AdjTargets<T, D, N, P, M + 1, LO, K>::template run<ASUB, HSUB, KS>(a, asub, hc, hsub, dxs, dxf, dxp, gdxk,
+                                                                                 gdxf, gpre);
     }
 };
 
@@ -394,11 +434,29 @@ __device__ __forceinline__ void read_increments(const T *sdx, int tt, const int 
     for (int j = 0; j < P; ++j) dxp[j] = sdx[tt * KS * D + u[j]];
 }
 
+// scaled increments of the K letters a0 .. a0 + K - 1 (zero beyond the alphabet); a0 is the same for a whole wave
+template <typename T, int D, int K, int KS, int FQ, int FK>
+__device__ __forceinline__ void read_first_level(const T *sdx, int tt, int a0, T (&dxf)[FQ][FK]) {
+    static_assert(FQ == KS && FK == K, "only called where the first level is split");
+#pragma unroll
+    for (int q = 0; q < KS; ++q)
+#pragma unroll
+        for (int i = 0; i < K; ++i) dxf[q][i] = a0 + i < D ? sdx[(tt * KS + q) * D + a0 + i] : T(0);
+}
+
 constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2) : 1; }
 
 template <int D, int N, int P, int ELEM = 4>
 struct Geometry {
-    static constexpr int kLanes = ipow(D, P);
+    // A lane holds kK children of its prefix: all D, or fewer where the first level below the prefix is split
+    // between kParts lanes (split_children).  The lanes of a part are padded to whole waves, so the part, and with
+    // it the letters of the lane's children, is the same for all lanes of a wave.
+    static constexpr int kK = split_children(D, N, P);
+    static constexpr bool kSplit = kK < D;
+    static constexpr int kParts = (D + kK - 1) / kK;
+    static constexpr int kPrefixes = ipow(D, P);
+    static constexpr int kPartLanes = kSplit ? (kPrefixes + kWave - 1) / kWave * kWave : kPrefixes;
+    static constexpr int kLanes = kSplit ? kParts * kPartLanes : kPrefixes;
     // A unit needs kUnitWaves waves.  Up to sixteen of them form one block; a larger unit is spread over
     // kUnitBlocks blocks (its lanes never talk to each other inside a sweep; the per-increment sums of the
     // backward then meet in memory).  Such shapes are swept in one piece, without time chunks.
@@ -407,9 +465,10 @@ struct Geometry {
     // each lane 128 registers, which the reverse sweep of such a shape overflows), four from 160 values on (one
     // wave per SIMD: 512 registers, the upper half reached through copies); a unit that needs several blocks
     // anyway takes the smaller block from a smaller sub-trie on
-    static constexpr int kSubTrie = trie_size(D, N - P);
+    static constexpr int kSubTrie = sub_size(D, kK, N - P);
     static constexpr int kMaxWaves32 =
-        kSubTrie > 160 ? 4 : (kSubTrie > 40 || (kUnitWaves > 16 && kSubTrie > 30)) ? 8 : 16;
+        (kSubTrie > 160 || (kSplit && kSubTrie > 128)) ? 4
+        : (kSubTrie > 40 || (kUnitWaves > 16 && kSubTrie > 30)) ? 8 : 16;
     // fp64 doubles the registers of a lane's state.  Where the unit is spread over several blocks anyway (or,
     // with three levels below the prefix, would fill more than eight waves), the blocks shrink until the state
     // fits: the reverse sweeps of these shapes spilled 200 to 400 registers to memory in blocks of eight or
@@ -419,11 +478,14 @@ struct Geometry {
         !kSplit64 ? kMaxWaves32
         : (kSubTrie >= 72 || N - P >= 3 || (kSubTrie >= 56 && P >= 6)) ? 4
         : kSubTrie >= 30 ? (kMaxWaves32 < 8 ? kMaxWaves32 : 8) : kMaxWaves32;
-    static constexpr int kWaves = kUnitWaves < kMaxWaves ? kUnitWaves : kMaxWaves;
+    // a unit of several blocks deals its waves out evenly (18 waves: three blocks of six, not 8 + 8 + 2 with six
+    // waves that sweep nothing)
+    static constexpr int kUnitBlocks = (kUnitWaves + kMaxWaves - 1) / kMaxWaves;
+    static constexpr int kWaves = (kUnitWaves + kUnitBlocks - 1) / kUnitBlocks;
     static constexpr int kBlock = kWaves * kWave;
-    static constexpr int kUnitBlocks = (kUnitWaves + kWaves - 1) / kWaves;
-    static constexpr int kFwdSub = trie_size(D, N - P);    // sub-trie levels P+1..N
-    static constexpr int kASub = trie_size(D, N - 1 - P);  // levels P+1..N-1
+    static constexpr int kFwdSub = sub_size(D, kK, N - P);    // sub-trie levels P+1..N
+    static constexpr int kASub = sub_size(D, kK, N - 1 - P);  // levels P+1..N-1
+    static_assert(!kSplit || kUnitBlocks > 1, "a split first level is only built for units swept in one piece");
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
         int64_t o = 0, w = 1;
         for (int i = 1; i < k; ++i) {
@@ -450,8 +512,10 @@ __device__ __forceinline__ void prefix_letters(int pu, int (&u)[P]) {
 // lane state <-> dense layout in memory
 // ---------------------------------------------------------------------------------------------
 // Reads the chain a[1..P] and the sub-trie levels P+1..TOP of prefix pu from a dense-layout row.
-template <typename T, int D, int P, int TOP, int SUB>
-__device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bool active, T (&a)[P + 1], T (&sub)[SUB]) {
+// K < D: the lane holds the children a0 .. a0 + K - 1 of its prefix only (those beyond the alphabet read as zero).
+template <typename T, int D, int P, int TOP, int SUB, int K = D>
+__device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bool active, T (&a)[P + 1], T (&sub)[SUB],
+                                           int a0 = 0) {
     using G = Geometry<D, TOP, P>;
     int rest = 1;
 #pragma unroll
@@ -461,16 +525,20 @@ __device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bo
     }
     static_for<1, TOP - P + 1>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        constexpr int width = ipow(D, k);
-        constexpr int off = trie_size(D, k - 1);
-        const T *src = row + G::level_off(P + k) + (int64_t)pu * width;
+        constexpr int below = ipow(D, k - 1);  // words of this level below one child
+        constexpr int off = sub_size(D, K, k - 1);
+        const T *src = row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
 #pragma unroll
-        for (int i = 0; i < width; ++i) sub[off + i] = active ? src[i] : T(0);
+        for (int i = 0; i < K * below; ++i) {
+            const bool have = K == D || a0 + i / below < D;
+            sub[off + i] = (active && have) ? src[i] : T(0);
+        }
     });
 }
 
-template <typename T, int D, int P, int TOP, int SUB>
-__device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T (&a)[P + 1], const T (&sub)[SUB]) {
+template <typename T, int D, int P, int TOP, int SUB, int K = D>
+__device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T (&a)[P + 1], const T (&sub)[SUB],
+                                            int a0 = 0) {
     using G = Geometry<D, TOP, P>;
     // Every lane writes its chain values: lanes that share a chain node computed it with the same
     // operations, so they store identical bits, and no branch is needed.
@@ -482,11 +550,12 @@ __device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T
     }
     static_for<1, TOP - P + 1>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
-        constexpr int width = ipow(D, k);
-        constexpr int off = trie_size(D, k - 1);
-        T *dst = row + G::level_off(P + k) + (int64_t)pu * width;
+        constexpr int below = ipow(D, k - 1);
+        constexpr int off = sub_size(D, K, k - 1);
+        T *dst = row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
 #pragma unroll
-        for (int i = 0; i < width; ++i) dst[i] = sub[off + i];
+        for (int i = 0; i < K * below; ++i)
+            if (K == D || a0 + i / below < D) dst[i] = sub[off + i];
     });
 }
 
@@ -636,9 +705,15 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
     constexpr int KS = N - P;
     const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
     T *sdx = sdx_all[part];
-    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
+    // first level split between lanes: pu counts (part of the children, prefix); pp is the prefix
+    constexpr int KF = G::kK, FQ = G::kSplit ? KS : 1, FK = G::kSplit ? KF : 1;
+    const int spart = G::kSplit ? pu / G::kPartLanes : 0;
+    const int pp = G::kSplit ? pu - spart * G::kPartLanes : pu;
+    const int a0 = spart * KF;
+    const bool active = G::kSplit ? (pp < G::kPrefixes && spart < G::kParts)
+                                  : ((G::kLanes == G::kBlock) || pu < G::kLanes);
     int u[P];
-    prefix_letters<D, P>(active ? pu : 0, u);
+    prefix_letters<D, P>(active ? pp : 0, u);
 
     const int groups = chunks / GW;  // blocks per row
     const int64_t blk = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
@@ -680,21 +755,32 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             // two register sets of increments: the LDS reads of the next step are issued before the
             // arithmetic of the current one, so their latency hides behind it
             T dxs0[KS][D], dxp0[P], dxs1[KS][D], dxp1[P];
-            read_increments<T, D, P, KS>(sdx, 0, u, dxs0, dxp0);
+            T dxf0[FQ][FK], dxf1[FQ][FK];
+            auto read = [&](int at, T (&dxs)[KS][D], T (&dxp)[P], T (&dxf)[FQ][FK]) {
+                read_increments<T, D, P, KS>(sdx, at, u, dxs, dxp);
+                if constexpr (G::kSplit) read_first_level<T, D, KF, KS>(sdx, at, a0, dxf);
+            };
+            auto step = [&](const T (&dxs)[KS][D], const T (&dxp)[P], const T (&dxf)[FQ][FK]) {
+                if constexpr (G::kSplit)
+                    StepTargets<T, D, P, N, false, BOUND, KF>::template run<G::kFwdSub, KS>(a, sub, dxs, dxf, dxp);
+                else
+                    StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs, dxs, dxp);
+            };
+            read(0, dxs0, dxp0, dxf0);
             int tt = 0;
             for (; tt + 1 < nt; tt += 2) {
-                read_increments<T, D, P, KS>(sdx, tt + 1, u, dxs1, dxp1);
-                StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
-                read_increments<T, D, P, KS>(sdx, tt + 2 < nt ? tt + 2 : tt + 1, u, dxs0, dxp0);
-                StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs1, dxp1);
+                read(tt + 1, dxs1, dxp1, dxf1);
+                step(dxs0, dxp0, dxf0);
+                read(tt + 2 < nt ? tt + 2 : tt + 1, dxs0, dxp0, dxf0);
+                step(dxs1, dxp1, dxf1);
             }
-            if (tt < nt) StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs0, dxp0);
+            if (tt < nt) step(dxs0, dxp0, dxf0);
         }
     }
     if constexpr (N - 1 >= P) {
         // the chunk's own signature below the top level, kept for the backward of the same call
         if (chunk_low != nullptr && active)
-            store_state<T, D, P, N - 1, G::kFwdSub>(chunk_low + (row * chunks + c) * G::kLowSize, pu, a, sub);
+            store_state<T, D, P, N - 1, G::kFwdSub, KF>(chunk_low + (row * chunks + c) * G::kLowSize, pp, a, sub, a0);
     }
     if constexpr (GW > 1) {
         const SubWords<D, P> sw(u);
@@ -710,7 +796,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
         }
         if (part == 0 && active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
     } else {
-        if (active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
+        if (active) store_state<T, D, P, N, G::kFwdSub, KF>(out + blk * G::kSigSize, pp, a, sub, a0);
     }
 }
 
@@ -843,13 +929,14 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 // lane-private partial sums, so only the lane whose remaining prefix letters are zero starts from it.
 template <typename T, int D, int N, int P>
 __device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu, bool active, T (&hc)[P + 1],
-                                             T (&hsub)[Geometry<D, N, P>::kFwdSub]) {
+                                             T (&hsub)[Geometry<D, N, P>::kFwdSub], int a0 = 0) {
     using G = Geometry<D, N, P>;
-    load_state<T, D, P, N, G::kFwdSub>(grow, pu, active, hc, hsub);
+    load_state<T, D, P, N, G::kFwdSub, G::kK>(grow, pu, active, hc, hsub, a0);
     int rest = 1;
 #pragma unroll
     for (int j = P; j >= 1; --j) {
-        if (pu % rest != 0) hc[j] = T(0);
+        // (of the lanes that split the children of one prefix, the first one)
+        if (pu % rest != 0 || a0 != 0) hc[j] = T(0);
         rest *= D;
     }
     hc[0] = T(0);
@@ -1047,8 +1134,8 @@ template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, int BO
 __device__ __forceinline__ void dense_backward_body(
     const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig, const T *__restrict__ edgeA,
     const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
-    const int pu,   // prefix of the thread
-    const int tid,  // index of the thread within its block
+    const int pu_unit,  // index of the thread within its unit (its prefix, unless the first level is split)
+    const int tid,      // index of the thread within its block
     T (&sdx)[BackwardShape<T, D, N, P>::kStage],
     T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
     T (&cells)[BackwardShape<T, D, N, P>::kCells]) {
@@ -1060,7 +1147,13 @@ __device__ __forceinline__ void dense_backward_body(
     constexpr bool kToPath = CHUNKED && !ACCUMULATE;  // writes the path gradient itself (see the tile flush)
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;  // within the block
-    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
+    // first level split between lanes: pu_unit counts (part of the children, prefix); pu is the prefix
+    constexpr int KF = G::kK, FQ = G::kSplit ? KS : 1, FK = G::kSplit ? KF : 1;
+    const int spart = G::kSplit ? pu_unit / G::kPartLanes : 0;
+    const int pu = G::kSplit ? pu_unit - spart * G::kPartLanes : pu_unit;
+    const int a0 = spart * KF;
+    const bool active = G::kSplit ? (pu < G::kPrefixes && spart < G::kParts)
+                                  : ((G::kLanes == G::kBlock) || pu < G::kLanes);
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
     // chain terms through LDS (see BackwardShape): the lane's cells start at zero
@@ -1087,7 +1180,7 @@ __device__ __forceinline__ void dense_backward_body(
     T a[P + 1], hc[P + 1];
     T asub[kAS];
     T hsub[G::kFwdSub];
-    load_adjoint<T, D, N, P>(grow, pu, active, hc, hsub);
+    load_adjoint<T, D, N, P>(grow, pu, active, hc, hsub, a0);
     if constexpr (CHUNKED) {
         load_state<T, D, P, N - 1, kAS>(edgeA + unit * G::kLowSize, pu, active, a, asub);
         // adjoint at the right edge of the chunk: the upstream gradient contracted with the signature of
@@ -1095,7 +1188,7 @@ __device__ __forceinline__ void dense_backward_body(
         const SubWords<D, P> sw(u);
         contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
     } else {
-        load_state<T, D, P, N - 1, kAS>(sig + row * G::kSigSize, pu, active, a, asub);
+        load_state<T, D, P, N - 1, kAS, KF>(sig + row * G::kSigSize, pu, active, a, asub, a0);
     }
     a[0] = T(1);
     // onehot[j][k] = 1 when the j-th letter of the lane's prefix is k (kept in registers only where
@@ -1119,18 +1212,32 @@ __device__ __forceinline__ void dense_backward_body(
         lds_barrier();
         stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, tid);
         lds_barrier();
-        auto step = [&](int tt, const T (&dxs)[KS][D], const T (&dxp)[P]) {
+        auto step = [&](int tt, const T (&dxs)[KS][D], const T (&dxp)[P], const T (&dxf)[FQ][FK]) {
             // A_t = A_{t+1} (x) exp(-dx_t), levels < N
-            if constexpr (N > 1) StepTargets<T, D, P, N - 1, true>::template run<kAS, KS>(a, asub, dxs, dxp);
+            if constexpr (N > 1) {
+                if constexpr (G::kSplit)
+                    StepTargets<T, D, P, N - 1, true, 0, KF>::template run<kAS, KS>(a, asub, dxs, dxf, dxp);
+                else
+                    StepTargets<T, D, P, N - 1, true>::template run<kAS, KS>(a, asub, dxs, dxs, dxp);
+            }
             T gdxk[KS][D], gpre[P];
+            T gdxf[FQ][FK];
+#pragma unroll
+            for (int q = 0; q < FQ; ++q)
+#pragma unroll
+                for (int i = 0; i < FK; ++i) gdxf[q][i] = T(0);
 #pragma unroll
             for (int q = 0; q < KS; ++q)
 #pragma unroll
                 for (int k = 0; k < D; ++k) gdxk[q][k] = T(0);
 #pragma unroll
             for (int j = 0; j < P; ++j) gpre[j] = T(0);
-            AdjTargets<T, D, N, P, 1, BOUND>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxp, gdxk,
-                                                                                gpre);
+            if constexpr (G::kSplit)
+                AdjTargets<T, D, N, P, 1, BOUND, KF>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxf, dxp,
+                                                                                        gdxk, gdxf, gpre);
+            else
+                AdjTargets<T, D, N, P, 1, BOUND>::template run<kAS, G::kFwdSub, KS>(a, asub, hc, hsub, dxs, dxs, dxp,
+                                                                                    gdxk, gdxk, gpre);
             // letter k collects the sub-trie sums (with the 1/(q+1) of their increments) and the chain
             // positions whose letter is k
             T tot[D];
@@ -1169,6 +1276,28 @@ __device__ __forceinline__ void dense_backward_body(
                     const int letter = base + row_letter<DP>(lane);
                     if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
                 }
+                if constexpr (G::kSplit) {
+                    // The lane's own children carry the letters a0 .. a0 + K - 1, the same for the whole wave.  Their
+                    // row sums are added to the cells just written: the cell depends on the part, and a register
+                    // array cannot be indexed at run time.  (The LDS operations of a wave complete in order.)
+                    constexpr int KP = KF <= 2 ? 2 : KF <= 4 ? 4 : 8;
+                    static_assert(KF <= 8, "one pass of exchanges holds eight letters");
+                    T padded[KP];
+#pragma unroll
+                    for (int k = 0; k < KP; ++k) {
+                        T v = T(0);
+                        if (k < KF) {
+                            v = gdxf[0][k < FK ? k : 0];
+#pragma unroll
+                            for (int q = 1; q < FQ; ++q) v = fmad<T>(gdxf[q][k < FK ? k : 0], rcp<T>(q + 1), v);
+                        }
+                        padded[k] = v;
+                    }
+                    const T r = row_totals<T, KP>(padded, lane);
+                    const int li = row_letter<KP>(lane);
+                    if (row_writer<KP>(lane) && li < KF && a0 + li < D)
+                        sg[wave * 4 + (lane >> 4)][tt * D + a0 + li] += r;
+                }
             } else {
 #pragma unroll
                 for (int k = 0; k < D; ++k) {
@@ -1186,21 +1315,28 @@ __device__ __forceinline__ void dense_backward_body(
         if constexpr (sizeof(T) == 4) {
             // two register sets of increments, so the LDS reads of the next step hide behind the current one
             T dxs0[KS][D], dxp0[P], dxs1[KS][D], dxp1[P];
+            T dxf0[FQ][FK], dxf1[FQ][FK];
+            auto read = [&](int at, T (&dxs)[KS][D], T (&dxp)[P], T (&dxf)[FQ][FK]) {
+                read_increments<T, D, P, KS>(sdx, at, u, dxs, dxp);
+                if constexpr (G::kSplit) read_first_level<T, D, KF, KS>(sdx, at, a0, dxf);
+            };
             int tt = nt - 1;
-            read_increments<T, D, P, KS>(sdx, tt, u, dxs0, dxp0);
+            read(tt, dxs0, dxp0, dxf0);
             for (; tt >= 1; tt -= 2) {
-                read_increments<T, D, P, KS>(sdx, tt - 1, u, dxs1, dxp1);
-                step(tt, dxs0, dxp0);
-                read_increments<T, D, P, KS>(sdx, tt - 2 >= 0 ? tt - 2 : 0, u, dxs0, dxp0);
-                step(tt - 1, dxs1, dxp1);
+                read(tt - 1, dxs1, dxp1, dxf1);
+                step(tt, dxs0, dxp0, dxf0);
+                read(tt - 2 >= 0 ? tt - 2 : 0, dxs0, dxp0, dxf0);
+                step(tt - 1, dxs1, dxp1, dxf1);
             }
-            if (tt == 0) step(0, dxs0, dxp0);
+            if (tt == 0) step(0, dxs0, dxp0, dxf0);
         } else {
             // fp64 state fills the register file: one set of increments
             for (int tt = nt - 1; tt >= 0; --tt) {
                 T dxs[KS][D], dxp[P];
+                T dxf[FQ][FK];
                 read_increments<T, D, P, KS>(sdx, tt, u, dxs, dxp);
-                step(tt, dxs, dxp);
+                if constexpr (G::kSplit) read_first_level<T, D, KF, KS>(sdx, tt, a0, dxf);
+                step(tt, dxs, dxp, dxf);
             }
         }
         lds_barrier();
@@ -1294,7 +1430,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(47, 11, 3, 2, 2, 1) X(48, 12, 3, 2, 2, 1) X(49, 13, 3, 2, 2, 1) X(50, 14, 3, 2, 2, 1) \
     X(51, 15, 3, 2, 2, 1) X(52, 16, 3, 2, 2, 1) X(53, 9, 4, 2, 3, 2) X(54, 10, 4, 2, 3, 2) \
     X(55, 11, 4, 2, 3, 2) X(56, 12, 4, 2, 3, 2) X(57, 13, 4, 2, 3, 2) X(58, 14, 4, 2, 3, 2) \
-    X(59, 15, 4, 2, 3, 2) X(60, 16, 4, 3, 3, 2) X(61, 9, 5, 3, 3, 3) X(62, 10, 5, 3, 3, 3) \
+    X(59, 15, 4, 2, 3, 2) X(60, 16, 4, 2, 3, 2) X(61, 9, 5, 3, 3, 3) X(62, 10, 5, 3, 3, 3) \
     X(63, 11, 5, 3, 3, 3) X(64, 12, 5, 3, 3, 3) X(65, 2, 7, 5, 6, 5) X(66, 3, 7, 4, 5, 4) \
     X(67, 4, 7, 4, 5, 4) X(68, 3, 8, 5, 6, 5) X(69, 2, 9, 6, 8, 7) X(70, 2, 10, 6, 8, 7) \
     X(71, 17, 2, 1, 1, 1) X(72, 18, 2, 1, 1, 1) X(73, 19, 2, 1, 1, 1) X(74, 20, 2, 1, 1, 1) \
@@ -1327,16 +1463,21 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(178, 3, 12, 9, 6, 6) X(179, 4, 10, 7, 6, 6) X(180, 4, 11, 8, 6, 6) X(181, 5, 8, 6, 5, 5) \
     X(182, 5, 9, 7, 5, 5) X(183, 6, 8, 6, 5, 5) X(184, 7, 8, 6, 5, 5) X(185, 9, 6, 4, 4, 3) \
     X(186, 10, 6, 4, 4, 3) X(187, 11, 6, 4, 4, 3) X(188, 12, 6, 4, 4, 3) X(189, 13, 5, 3, 3, 3) \
-    X(190, 14, 5, 3, 3, 3) X(191, 15, 5, 3, 3, 3) X(192, 16, 5, 4, 4, 3) X(193, 17, 4, 3, 3, 2) \
-    X(194, 18, 4, 3, 3, 2) X(195, 19, 4, 3, 3, 2) X(196, 20, 4, 3, 3, 2) X(197, 21, 4, 3, 3, 2) \
-    X(198, 22, 4, 3, 3, 2) X(199, 23, 4, 3, 3, 2) X(200, 24, 4, 3, 3, 2) X(201, 25, 4, 3, 3, 2) \
-    X(202, 26, 4, 3, 3, 2) X(203, 27, 4, 3, 3, 2) X(204, 28, 4, 3, 3, 2) X(205, 29, 4, 3, 3, 2) \
-    X(206, 30, 4, 3, 3, 2) X(207, 31, 4, 3, 3, 2) X(208, 32, 4, 3, 3, 2) \
+    X(190, 14, 5, 3, 3, 3) X(191, 15, 5, 3, 3, 3) X(192, 16, 5, 3, 3, 3) X(193, 17, 4, 2, 3, 2) \
+    X(194, 18, 4, 2, 3, 2) X(195, 19, 4, 2, 3, 2) X(196, 20, 4, 2, 3, 2) X(197, 21, 4, 2, 3, 2) \
+    X(198, 22, 4, 2, 3, 2) X(199, 23, 4, 2, 3, 2) X(200, 24, 4, 2, 3, 2) X(201, 25, 4, 2, 3, 2) \
+    X(202, 26, 4, 2, 3, 2) X(203, 27, 4, 2, 3, 2) X(204, 28, 4, 2, 3, 2) X(205, 29, 4, 2, 3, 2) \
+    X(206, 30, 4, 2, 3, 2) X(207, 31, 4, 2, 3, 2) X(208, 32, 4, 2, 3, 2) \
     X(209, 9, 4, 3, 3, 2) X(210, 10, 4, 3, 3, 2) X(211, 11, 4, 3, 3, 2) X(212, 12, 4, 3, 3, 2) \
     X(213, 13, 4, 3, 3, 2) X(214, 14, 4, 3, 3, 2) X(215, 15, 4, 3, 3, 2) X(216, 9, 5, 4, 4, 3) \
     X(217, 10, 5, 4, 4, 3) X(218, 11, 5, 4, 4, 3) X(219, 12, 5, 4, 4, 3) X(220, 13, 5, 4, 4, 3) \
     X(221, 14, 5, 4, 4, 3) X(222, 15, 5, 4, 4, 3) X(223, 9, 6, 5, 5, 4) X(224, 10, 6, 5, 5, 4) \
-    X(225, 11, 6, 5, 5, 4) X(226, 12, 6, 5, 5, 4)
+    X(225, 11, 6, 5, 5, 4) X(226, 12, 6, 5, 5, 4) \
+    X(227, 16, 4, 3, 3, 2) X(228, 16, 5, 4, 4, 3) X(229, 17, 4, 3, 3, 2) X(230, 18, 4, 3, 3, 2) \
+    X(231, 19, 4, 3, 3, 2) X(232, 20, 4, 3, 3, 2) X(233, 21, 4, 3, 3, 2) X(234, 22, 4, 3, 3, 2) \
+    X(235, 23, 4, 3, 3, 2) X(236, 24, 4, 3, 3, 2) X(237, 25, 4, 3, 3, 2) X(238, 26, 4, 3, 3, 2) \
+    X(239, 27, 4, 3, 3, 2) X(240, 28, 4, 3, 3, 2) X(241, 29, 4, 3, 3, 2) X(242, 30, 4, 3, 3, 2) \
+    X(243, 31, 4, 3, 3, 2) X(244, 32, 4, 3, 3, 2)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.
@@ -1365,7 +1506,7 @@ constexpr VariantInfo variant_info() {
                        LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
                        {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
                         G64::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
-                       trie_size(D, N - P) <= 132};
+                       !G::kSplit && trie_size(D, N - P) <= 132};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1650,7 +1791,7 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             for (int j = i + 1; j < kNumVariants; ++j) later = later || (kVariants[j].d == d && kVariants[j].depth == depth);
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
             if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
-            // the short prefixes of the wide alphabets hold 90 to 240 values per lane: fp64 up to 132 (d = 11)
+            // the short prefixes of the wide alphabets hold 68 to 240 values per lane: fp64 up to 132 (d = 11, no split)
             if (later && elem == 8 && !v.fp64_fits) continue;
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];

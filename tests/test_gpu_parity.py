@@ -1006,11 +1006,15 @@ def test_per_word_kernels_on_shapes_that_have_a_tiled_kernel(ps, set_option, dty
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("d,depth,B,L", [(9, 4, 64, 150), (12, 4, 64, 150), (13, 4, 64, 150), (15, 4, 64, 150),
                                          (9, 5, 12, 150), (12, 5, 12, 150), (13, 5, 12, 150), (15, 5, 12, 40),
-                                         (9, 6, 6, 40), (12, 6, 2, 24)])
+                                         (9, 6, 6, 40), (12, 6, 2, 24),
+                                         (16, 4, 64, 40), (17, 4, 64, 40), (20, 4, 32, 40), (23, 4, 32, 40),
+                                         (29, 4, 16, 24), (32, 4, 16, 24), (16, 5, 8, 24)])
 def test_wide_alphabets_with_enough_rows_for_the_short_prefix(ps, dtype, d, depth, B, L):
-    """d = 9..15 at depth 4 and 5 and d = 9..12 at depth 6 are compiled twice: lanes on prefixes of length depth - 2 (90 to 240 values per lane,
-    fp32 only, taken when the rows fill the device) and of length depth - 1 (fp64, few rows).  Enough rows here for
-    the first kind; the checker runs on two of them."""
+    """d = 9..32 at depth 4, 9..16 at depth 5 and 9..12 at depth 6 are compiled twice: lanes on prefixes of length
+    depth - 2 (68 to 240 values per lane, taken in fp32 when the rows fill the device; from d = 16 on the children
+    of a prefix are split between several lanes, the last of which may hold fewer: 17 = 6 + 6 + 5, 23 = 5 x 4 + 3,
+    29 = 7 x 4 + 1) and of length depth - 1 (fp64 from d = 12 on, few rows).  Enough rows here for the first kind; the
+    checker runs on two of them."""
     path = brownian_path(B, L, d, seed=800 + d + depth)
     x = path.to(dtype).to(DEV).requires_grad_(True)
     out = ps.Signature(depth=depth)(x)
