@@ -65,13 +65,15 @@ constexpr int trie_size(int D, int k) { return k <= 0 ? 0 : ipow(D, k) + trie_si
 // values on the first k levels below a lane's prefix when the lane holds K children of the prefix (all D of them
 // unless the first level is split between several lanes) and every child's complete sub-trie
 constexpr int sub_size(int D, int K, int k) { return k <= 0 ? 0 : K * ipow(D, k - 1) + sub_size(D, K, k - 1); }
-// Children of the prefix that one lane holds.  The widest alphabets at depth 4 and 5 split them between lanes: with
-// all D children a lane would hold D + D^2 = 272 values and more, with the next longer prefix only D.
+// Children of the prefix that one lane holds.  The widest alphabets (d = 16..32 at depth 4, 12..16 at depth 5) split
+// them between lanes: with all D children a lane would hold D + D^2 = 156 to 1056 values, with the next longer
+// prefix only D.
 // Chosen by an estimate of the useful share of a lane's instructions: K / (K + 1.5) for the chain, the per-letter
 // sums and the reduction that every lane pays whatever K is, times the share of child slots in use (the last lane
 // of a prefix may hold fewer than K), within K * (D + 1) <= 136 values.
 constexpr int split_children(int D, int N, int P) {
-    if (!(D >= 16 && D <= 32 && P == N - 2 && (N == 4 || (N == 5 && D == 16)))) return D;
+    // (d = 13 at depth 5 measured slower split, 24.7 against 32.3 TFLOP/s, and keeps all its children in one lane)
+    if (!(P == N - 2 && ((N == 4 && D >= 16 && D <= 32) || (N == 5 && D >= 12 && D <= 16 && D != 13)))) return D;
     int best = 2;
     long best_num = 0, best_den = 1;
     for (int k = 2; k * (D + 1) <= 136 && k <= 8; ++k) {
