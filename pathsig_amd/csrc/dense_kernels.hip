@@ -65,7 +65,8 @@ constexpr int trie_size(int D, int k) { return k <= 0 ? 0 : ipow(D, k) + trie_si
 // values on the first k levels below a lane's prefix when the lane holds K children of the prefix (all D of them
 // unless the first level is split between several lanes) and every child's complete sub-trie
 constexpr int sub_size(int D, int K, int k) { return k <= 0 ? 0 : K * ipow(D, k - 1) + sub_size(D, K, k - 1); }
-// Children of the prefix that one lane holds.  The widest alphabets (d = 16..32 at depth 4, 12..16 at depth 5) split
+// Children of the prefix that one lane holds.  The widest alphabets (d = 28..48 at depth 3, 16..32 at depth 4, 12..16
+// at depth 5) split
 // them between lanes: with all D children a lane would hold D + D^2 = 156 to 1056 values, with the next longer
 // prefix only D.
 // Chosen by an estimate of the useful share of a lane's instructions: K / (K + 1.5) for the chain, the per-letter
@@ -73,7 +74,9 @@ constexpr int sub_size(int D, int K, int k) { return k <= 0 ? 0 : K * ipow(D, k 
 // of a prefix may hold fewer than K), within K * (D + 1) <= 136 values.
 constexpr int split_children(int D, int N, int P) {
     // (d = 13 at depth 5 measured slower split, 24.7 against 32.3 TFLOP/s, and keeps all its children in one lane)
-    if (!(P == N - 2 && ((N == 4 && D >= 16 && D <= 32) || (N == 5 && D >= 12 && D <= 16 && D != 13)))) return D;
+    if (!(P == N - 2 && ((N == 3 && D >= 28 && D <= 48) || (N == 4 && D >= 16 && D <= 32) ||
+                         (N == 5 && D >= 12 && D <= 16 && D != 13))))
+        return D;
     int best = 2;
     long best_num = 0, best_den = 1;
     for (int k = 2; k * (D + 1) <= 136 && k <= 8; ++k) {
@@ -451,13 +454,14 @@ constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2
 template <int D, int N, int P, int ELEM = 4>
 struct Geometry {
     // A lane holds kK children of its prefix: all D, or fewer where the first level below the prefix is split
-    // between kParts lanes (split_children).  The lanes of a part are padded to whole waves, so the part, and with
-    // it the letters of the lane's children, is the same for all lanes of a wave.
+    // between kParts lanes (split_children).  The lanes of a part are padded to whole rows of sixteen lanes (the unit
+    // of the per-letter sums), so the part, and with it the letters of the lane's children, is the same for all lanes
+    // of such a row.
     static constexpr int kK = split_children(D, N, P);
     static constexpr bool kSplit = kK < D;
     static constexpr int kParts = (D + kK - 1) / kK;
     static constexpr int kPrefixes = ipow(D, P);
-    static constexpr int kPartLanes = kSplit ? (kPrefixes + kWave - 1) / kWave * kWave : kPrefixes;
+    static constexpr int kPartLanes = kSplit ? (kPrefixes + 15) / 16 * 16 : kPrefixes;
     static constexpr int kLanes = kSplit ? kParts * kPartLanes : kPrefixes;
     // A unit needs kUnitWaves waves.  Up to sixteen of them form one block; a larger unit is spread over
     // kUnitBlocks blocks (its lanes never talk to each other inside a sweep; the per-increment sums of the
@@ -487,7 +491,9 @@ struct Geometry {
     static constexpr int kBlock = kWaves * kWave;
     static constexpr int kFwdSub = sub_size(D, kK, N - P);    // sub-trie levels P+1..N
     static constexpr int kASub = sub_size(D, kK, N - 1 - P);  // levels P+1..N-1
-    static_assert(!kSplit || kUnitBlocks > 1, "a split first level is only built for units swept in one piece");
+    // swept in one piece, never cut into time chunks: units of several blocks, and units with split children (the
+    // products of chunk signatures are not written for them)
+    static constexpr bool kOnePiece = kUnitBlocks > 1 || kSplit;
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
         int64_t o = 0, w = 1;
         for (int i = 1; i < k; ++i) {
@@ -815,7 +821,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock * GW))
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
     __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
     using G = Geometry<D, N, P, sizeof(T)>;
-    static_assert(G::kUnitBlocks == 1 || (GW == 1 && !BOUNDED), "a unit of several blocks is swept one chunk to a block");
+    static_assert(!G::kOnePiece || (GW == 1 && !BOUNDED), "a unit of several blocks is swept one chunk to a block");
     const int tid = (int)threadIdx.x % G::kBlock;
     if constexpr (BOUNDED) {
         const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
@@ -1391,7 +1397,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     __shared__ T sg[BS::kSums][BS::kSumRow];
     __shared__ T cells[BS::kCells];
     using G = Geometry<D, N, P, sizeof(T)>;
-    static_assert(G::kUnitBlocks == 1 || (ACCUMULATE && !CHUNKED && !BOUNDED),
+    static_assert((G::kUnitBlocks == 1 || ACCUMULATE) && (!G::kOnePiece || (!CHUNKED && !BOUNDED)),
                   "a unit of several blocks is swept in one piece and adds its per-increment sums in memory");
     const int tid = (int)threadIdx.x;
     if constexpr (BOUNDED) {
@@ -1441,8 +1447,8 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(83, 29, 2, 1, 1, 1) X(84, 30, 2, 1, 1, 1) X(85, 31, 2, 1, 1, 1) X(86, 32, 2, 1, 1, 1) \
     X(87, 17, 3, 2, 2, 1) X(88, 18, 3, 2, 2, 1) X(89, 19, 3, 2, 2, 1) X(90, 20, 3, 2, 2, 1) \
     X(91, 21, 3, 2, 2, 1) X(92, 22, 3, 2, 2, 1) X(93, 23, 3, 2, 2, 1) X(94, 24, 3, 2, 2, 1) \
-    X(95, 25, 3, 2, 2, 1) X(96, 26, 3, 2, 2, 1) X(97, 27, 3, 2, 2, 1) X(98, 28, 3, 2, 2, 1) \
-    X(99, 29, 3, 2, 2, 1) X(100, 30, 3, 2, 2, 1) X(101, 31, 3, 2, 2, 1) X(102, 32, 3, 2, 2, 1) \
+    X(95, 25, 3, 2, 2, 1) X(96, 26, 3, 2, 2, 1) X(97, 27, 3, 2, 2, 1) X(98, 28, 3, 1, 2, 1) \
+    X(99, 29, 3, 1, 2, 1) X(100, 30, 3, 1, 2, 1) X(101, 31, 3, 1, 2, 1) X(102, 32, 3, 1, 2, 1) \
     X(103, 33, 2, 1, 1, 1) X(104, 34, 2, 1, 1, 1) X(105, 35, 2, 1, 1, 1) X(106, 36, 2, 1, 1, 1) \
     X(107, 37, 2, 1, 1, 1) X(108, 38, 2, 1, 1, 1) X(109, 39, 2, 1, 1, 1) X(110, 40, 2, 1, 1, 1) \
     X(111, 41, 2, 1, 1, 1) X(112, 42, 2, 1, 1, 1) X(113, 43, 2, 1, 1, 1) X(114, 44, 2, 1, 1, 1) \
@@ -1451,10 +1457,10 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(123, 53, 2, 1, 1, 1) X(124, 54, 2, 1, 1, 1) X(125, 55, 2, 1, 1, 1) X(126, 56, 2, 1, 1, 1) \
     X(127, 57, 2, 1, 1, 1) X(128, 58, 2, 1, 1, 1) X(129, 59, 2, 1, 1, 1) X(130, 60, 2, 1, 1, 1) \
     X(131, 61, 2, 1, 1, 1) X(132, 62, 2, 1, 1, 1) X(133, 63, 2, 1, 1, 1) X(134, 64, 2, 1, 1, 1) \
-    X(135, 33, 3, 2, 2, 1) X(136, 34, 3, 2, 2, 1) X(137, 35, 3, 2, 2, 1) X(138, 36, 3, 2, 2, 1) \
-    X(139, 37, 3, 2, 2, 1) X(140, 38, 3, 2, 2, 1) X(141, 39, 3, 2, 2, 1) X(142, 40, 3, 2, 2, 1) \
-    X(143, 41, 3, 2, 2, 1) X(144, 42, 3, 2, 2, 1) X(145, 43, 3, 2, 2, 1) X(146, 44, 3, 2, 2, 1) \
-    X(147, 45, 3, 2, 2, 1) X(148, 46, 3, 2, 2, 1) X(149, 47, 3, 2, 2, 1) X(150, 48, 3, 2, 2, 1) \
+    X(135, 33, 3, 1, 2, 1) X(136, 34, 3, 1, 2, 1) X(137, 35, 3, 1, 2, 1) X(138, 36, 3, 1, 2, 1) \
+    X(139, 37, 3, 1, 2, 1) X(140, 38, 3, 1, 2, 1) X(141, 39, 3, 1, 2, 1) X(142, 40, 3, 1, 2, 1) \
+    X(143, 41, 3, 1, 2, 1) X(144, 42, 3, 1, 2, 1) X(145, 43, 3, 1, 2, 1) X(146, 44, 3, 1, 2, 1) \
+    X(147, 45, 3, 1, 2, 1) X(148, 46, 3, 1, 2, 1) X(149, 47, 3, 1, 2, 1) X(150, 48, 3, 1, 2, 1) \
     X(151, 49, 3, 2, 2, 1) X(152, 50, 3, 2, 2, 1) X(153, 51, 3, 2, 2, 1) X(154, 52, 3, 2, 2, 1) \
     X(155, 53, 3, 2, 2, 1) X(156, 54, 3, 2, 2, 1) X(157, 55, 3, 2, 2, 1) X(158, 56, 3, 2, 2, 1) \
     X(159, 57, 3, 2, 2, 1) X(160, 58, 3, 2, 2, 1) X(161, 59, 3, 2, 2, 1) X(162, 60, 3, 2, 2, 1) \
@@ -1479,14 +1485,20 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(231, 19, 4, 3, 3, 2) X(232, 20, 4, 3, 3, 2) X(233, 21, 4, 3, 3, 2) X(234, 22, 4, 3, 3, 2) \
     X(235, 23, 4, 3, 3, 2) X(236, 24, 4, 3, 3, 2) X(237, 25, 4, 3, 3, 2) X(238, 26, 4, 3, 3, 2) \
     X(239, 27, 4, 3, 3, 2) X(240, 28, 4, 3, 3, 2) X(241, 29, 4, 3, 3, 2) X(242, 30, 4, 3, 3, 2) \
-    X(243, 31, 4, 3, 3, 2) X(244, 32, 4, 3, 3, 2)
+    X(243, 31, 4, 3, 3, 2) X(244, 32, 4, 3, 3, 2) \
+    X(245, 28, 3, 2, 2, 1) X(246, 29, 3, 2, 2, 1) X(247, 30, 3, 2, 2, 1) X(248, 31, 3, 2, 2, 1) \
+    X(249, 32, 3, 2, 2, 1) X(250, 33, 3, 2, 2, 1) X(251, 34, 3, 2, 2, 1) X(252, 35, 3, 2, 2, 1) \
+    X(253, 36, 3, 2, 2, 1) X(254, 37, 3, 2, 2, 1) X(255, 38, 3, 2, 2, 1) X(256, 39, 3, 2, 2, 1) \
+    X(257, 40, 3, 2, 2, 1) X(258, 41, 3, 2, 2, 1) X(259, 42, 3, 2, 2, 1) X(260, 43, 3, 2, 2, 1) \
+    X(261, 44, 3, 2, 2, 1) X(262, 45, 3, 2, 2, 1) X(263, 46, 3, 2, 2, 1) X(264, 47, 3, 2, 2, 1) \
+    X(265, 48, 3, 2, 2, 1)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.
 template <typename T, int D, int N, int PS>
 constexpr bool scan_fits() {
     using GS = Geometry<D, N, PS>;
-    if (N < 2 || GS::kUnitBlocks > 1) return false;
+    if (N < 2 || GS::kOnePiece) return false;
     const int64_t padded = RowStager<T, (int)GS::kLowSize, GS::kBlock>::kPadded;
     return (2 * padded + 2 * GS::kLowSize) * (int64_t)sizeof(T) + 1024 <= 160 * 1024;
 }
@@ -1505,9 +1517,9 @@ constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
     using G64 = Geometry<D, N, P, 8>;
     return VariantInfo{D, N, G::kUnitWaves * kWave, G::kUnitBlocks, G::kSigSize, G::kLowSize,
-                       LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1 && D <= 16,
-                       {G::kUnitBlocks == 1 && scan_fits<float, D, N, PS>(),
-                        G64::kUnitBlocks == 1 && scan_fits<double, D, N, PS>()},
+                       LetterBounds<D, P>::kUsable && !G::kOnePiece && D <= 16,
+                       {!G::kOnePiece && scan_fits<float, D, N, PS>(),
+                        !G64::kOnePiece && scan_fits<double, D, N, PS>()},
                        !G::kSplit && trie_size(D, N - P) <= 132};
 }
 
@@ -1578,7 +1590,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
-    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && !G::kOnePiece;
     const int64_t rows = shape.B * shape.W;
     if (bounds && !kBoundsOk) return hipErrorInvalidValue;
     if (chunks <= 1) {
@@ -1593,7 +1605,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            dim3(G::kBlock), 0, stream, path, sig, shape, 1);
         return hipGetLastError();
     }
-    if constexpr (G::kUnitBlocks > 1) {
+    if constexpr (G::kOnePiece) {
         return hipErrorNotSupported;  // such shapes are never cut into time chunks (dense_choice)
     } else {
     // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits;
@@ -1646,7 +1658,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
                         hipStream_t stream) {
     using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PS>;
-    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && G::kUnitBlocks == 1;
+    constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && !G::kOnePiece;
     const int64_t rows = shape.B * shape.W;
     // per-increment sums are added in memory for overlapping windows and for units spread over several blocks
     const bool accumulate = shape.windows != nullptr || G::kUnitBlocks > 1;
@@ -1674,7 +1686,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         profile_bracket(false, stream);
         return hipGetLastError();
     }
-    if constexpr (G::kUnitBlocks > 1 || !scan_fits<T, D, N, PS>()) {
+    if constexpr (G::kOnePiece || !scan_fits<T, D, N, PS>()) {
         // never cut into time chunks (dense_choice): shapes whose units take several blocks, rows too long for
         // the scan kernel's LDS in this type
         return hipErrorNotSupported;
@@ -1792,7 +1804,10 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             bool later = false;
             for (int j = i + 1; j < kNumVariants; ++j) later = later || (kVariants[j].d == d && kVariants[j].depth == depth);
             const int64_t max_chunks = (L - 1) / 16 < 1 ? 1 : ((L - 1) / 16 > 64 ? 64 : (L - 1) / 16);
-            if (later && rows * (v.block / kWave) * max_chunks < 1024) continue;
+            // (a shape that is not cut into chunks has its rows only; half a wave per SIMD is then enough to take it,
+            // the later entry being two to three times slower per coefficient)
+            const bool cut = v.chunks_ok[elem == 8 ? 1 : 0];
+            if (later && rows * (v.block / kWave) * (cut ? max_chunks : 1) < (cut ? 1024 : 512)) continue;
             // the short prefixes of the wide alphabets hold 68 to 240 values per lane: fp64 up to 132 (d = 11, no split)
             if (later && elem == 8 && !v.fp64_fits) continue;
         }

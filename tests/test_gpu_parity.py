@@ -1008,9 +1008,10 @@ def test_per_word_kernels_on_shapes_that_have_a_tiled_kernel(ps, set_option, dty
                                          (9, 5, 12, 150), (12, 5, 12, 150), (13, 5, 12, 150), (15, 5, 12, 40),
                                          (9, 6, 6, 40), (12, 6, 2, 24),
                                          (16, 4, 64, 40), (17, 4, 64, 40), (20, 4, 32, 40), (23, 4, 32, 40),
-                                         (29, 4, 16, 24), (32, 4, 16, 24), (16, 5, 8, 24)])
+                                         (29, 4, 16, 24), (32, 4, 16, 24), (16, 5, 8, 24),
+                                         (28, 3, 256, 40), (33, 3, 256, 24), (47, 3, 128, 24)])
 def test_wide_alphabets_with_enough_rows_for_the_short_prefix(ps, dtype, d, depth, B, L):
-    """d = 9..32 at depth 4, 9..16 at depth 5 and 9..12 at depth 6 are compiled twice: lanes on prefixes of length
+    """d = 28..48 at depth 3, 9..32 at depth 4, 9..16 at depth 5 and 9..12 at depth 6 are compiled twice: lanes on prefixes of length
     depth - 2 (68 to 240 values per lane, taken in fp32 when the rows fill the device; from d = 16 on the children
     of a prefix are split between several lanes, the last of which may hold fewer: 17 = 6 + 6 + 5, 23 = 5 x 4 + 3,
     29 = 7 x 4 + 1) and of length depth - 1 (fp64 from d = 12 on, few rows).  Enough rows here for the first kind; the
