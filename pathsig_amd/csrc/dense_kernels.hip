@@ -8,7 +8,9 @@
 // register and the increment of the step is the same for all lanes of the unit: there is no
 // inter-lane traffic and no barrier inside the time loop.  One "unit" = one (path, window, time chunk); its
 // D^P lanes fill ceil(D^P / 64) wavefronts of one workgroup (of several for the largest shapes), each of
-// which stages a tile of increments in LDS.
+// which stages a tile of increments in LDS.  For the widest alphabets the D children of a prefix (and their
+// sub-tries) are dealt to several lanes, K to a lane, so that a lane's state still fits the register file
+// (split_children); the letters of a lane's children are then the same for every row of sixteen lanes.
 //
 // Horner form of one step for target level m (every node is one FMA):
 //     tmp_j[w a] = S_j[w a] + (tmp_{j-1}[w] / (m - j + 1)) * dx[a],   j = 1..m-1,   tmp_0 = 1
