@@ -1522,7 +1522,7 @@ constexpr VariantInfo variant_info() {
                        LetterBounds<D, P>::kUsable && !G::kOnePiece && D <= 16,
                        {!G::kOnePiece && scan_fits<float, D, N, PS>(),
                         !G64::kOnePiece && scan_fits<double, D, N, PS>()},
-                       !G::kSplit && trie_size(D, N - P) <= 132};
+                       G::kSplit || trie_size(D, N - P) <= 132};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -1810,7 +1810,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             // the later entry being two to three times slower per coefficient)
             const bool cut = v.chunks_ok[elem == 8 ? 1 : 0];
             if (later && rows * (v.block / kWave) * (cut ? max_chunks : 1) < (cut ? 1024 : 512)) continue;
-            // the short prefixes of the wide alphabets hold 68 to 240 values per lane: fp64 up to 132 (d = 11, no split)
+            // the short prefixes of the wide alphabets hold 68 to 240 values per lane: fp64 up to 132 (d = 11) and
+            // wherever the children are split
             if (later && elem == 8 && !v.fp64_fits) continue;
         }
         const bool chunks_ok = v.chunks_ok[elem == 8 ? 1 : 0];
