@@ -1025,3 +1025,34 @@ def test_wide_alphabets_with_enough_rows_for_the_short_prefix(ps, dtype, d, dept
     want = TO.signature(path[idx], depth)
     assert rel_err(out.detach().cpu()[idx], want) < TOL[dtype]
     assert rel_err(grad.cpu()[idx], TO.signature_vjp(path[idx], G[idx], depth)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("d,depth,B", [(16, 4, 40), (17, 4, 40), (32, 3, 64), (15, 5, 6)])
+def test_projection_and_windows_through_split_children(ps, dtype, d, depth, B):
+    """Enough rows for the variants whose lanes split the children of a prefix: dense and Lyndon-projected, with
+    overlapping and degenerate windows, through the modules (forward keeps the dense signature) and through the
+    stateless pair of operators (the backward sweeps again).  The checker runs on two paths."""
+    L = 12
+    windows = [(0, 12), (2, 9), (5, 6), (7, 7), (3, 11)]
+    path = brownian_path(B, L, d, seed=820 + d) * 1.5
+    idx = torch.tensor([0, B - 1])
+    for proj in (None, ps.projections.lyndon(depth=depth, path_dim=d)):
+        sizes, codes = _plan(proj)
+        x = path.to(dtype).to(DEV).requires_grad_(True)
+        win = torch.tensor(windows, dtype=torch.int64, device=DEV)
+        mod = ps.Signature(depth=depth, projection=proj, windows=win)
+        out = mod(x)
+        G = randn(tuple(out.shape), seed=821)
+        (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+        want = TO.compute_signature(path[idx], depth, sizes, codes, windows)
+        want_grad = TO.signature_vjp(path[idx], G[idx], depth, sizes, codes, windows)
+        assert rel_err(out.detach().cpu()[idx], want) < TOL[dtype]
+        assert rel_err(grad.cpu()[idx], want_grad) < TOL[dtype]
+        args = (mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes, mod.use_windows,
+                mod._windows)
+        with torch.no_grad():
+            sig = torch.ops.pathsig.compute_signature(x, *args)
+            g2 = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)
+        assert torch.equal(sig, out.detach())
+        assert rel_err(g2.cpu()[idx], want_grad) < TOL[dtype]
