@@ -1,6 +1,6 @@
 """Throughput of the signature hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2 | --shape D,N[,B[,L]]] [--no-cpu]
 
 One step = one forward + backward pass of the operator over one synthetic batch that is already
 resident in HBM.  The default workload is the headline configuration (depth-6 signature of 128
@@ -226,6 +226,10 @@ def main():
                          "its idle power state (its shader clock idles near 100 MHz and takes far longer than W short "
                          "steps to reach 2.4 GHz); 0 switches it off")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--shape", default=None, metavar="D,N[,B[,L]]",
+                    help="instead of a named configuration: dense signature of depth N in D dimensions, forward + "
+                         "backward, B paths (default 128) of L points (default 512); the tables of per-shape timings "
+                         "are made with this")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true",
@@ -248,7 +252,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     dtype = torch.float32 if args.dtype == "f32" else torch.float64
-    index = int(args.config[1])
+    if args.shape:
+        parts = [int(v) for v in args.shape.split(",")]
+        d, depth = parts[0], parts[1]
+        B = parts[2] if len(parts) > 2 else 128
+        L = parts[3] if len(parts) > 3 else 512
+        args.config = "shape"
+        CONFIGS["shape"] = dict(op="sig", B=B, L=L, d=d, depth=depth, backward=True,
+                                desc=f"signature depth {depth} fwd+bwd, B={B} L={L} d={d}")
+    index = int(args.config[1]) if args.config != "shape" else 9
     wl = make_workload(args.config, dtype, index)
     cfg, mod, x, G = wl["cfg"], wl["mod"], wl["x"], wl["G"]
     B = cfg["B"]
