@@ -222,6 +222,11 @@ int sig_forward_t(const void *path, void *sig, int64_t B, int64_t L, int64_t d, 
     return PATHSIG_OK;
 }
 
+// bytes of the per-increment sums dL/d(dx): of the call's type, fp64 behind the word-per-lane backward
+size_t inc_buffer_bytes(size_t elem, int64_t B, int64_t L, int64_t d, bool words_kernel) {
+    return align_up((size_t)(B * (L - 1) * d) * (words_kernel ? sizeof(double) : elem));
+}
+
 template <typename T>
 int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void *grad_path, int64_t B, int64_t L,
                    int64_t d, int depth, const int64_t *level_sizes, const int64_t *codes, int64_t n_encoded,
@@ -242,7 +247,9 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
         return PATHSIG_ERR_ARGUMENT;
     }
     plan.keep = const_cast<void *>(kept);
-    const size_t inc_bytes = align_up((size_t)(B * (L - 1) * d) * sizeof(T));
+    const bool words_kernel = !dc.usable && !batch_backward_usable(sizeof(T), B, d, shape.W);
+    const bool batch_wide = !dc.usable && !words_kernel && batch_wide_sums(sizeof(T), plan);
+    const size_t inc_bytes = inc_buffer_bytes(sizeof(T), B, L, d, words_kernel || batch_wide);
     const size_t need = inc_bytes + (dc.usable ? dc.backward_workspace : 0);
     if (!workspace || workspace_bytes < need) {
         set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
@@ -287,22 +294,38 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
                                      extra + used, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
         if (wrote_path) return PATHSIG_OK;
+    } else if (words_kernel || batch_wide) {
+        // lanes on words, or lanes on paths with a great many words: the per-increment sums are kept in fp64 (one
+        // term per block of words and cell)
+        double *ginc64 = (double *)workspace;
+        e = launch_fill_zero<double>(ginc64, B * (L - 1) * d, stream);
+        if (e != hipSuccess) return launch_failed(e, "fill launch");
+        if (shape.W > 0 && plan.sig_size > 0) {
+            profile_bracket(true, stream);
+            if (words_kernel)
+                e = launch_words_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc64, shape, plan,
+                                             codes, stream);
+            else
+                e = launch_batch_backward<T, double>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc64, shape,
+                                                     plan, codes, stream);
+            profile_bracket(false, stream);
+            if (e != hipSuccess) return launch_failed(e, "backward launch");
+        }
+        e = launch_increments_to_path<double, T>(ginc64, (T *)grad_path, B, L, d, stream);
+        if (e != hipSuccess) return launch_failed(e, "path-gradient launch");
+        return PATHSIG_OK;
     } else {
         e = launch_fill_zero<T>(ginc, B * (L - 1) * d, stream);
         if (e != hipSuccess) return launch_failed(e, "fill launch");
         if (shape.W > 0 && plan.sig_size > 0) {
             profile_bracket(true, stream);
-            if (batch_backward_usable(sizeof(T), B, d, shape.W))
-                e = launch_batch_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan,
-                                             codes, stream);
-            else
-                e = launch_words_backward<T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan,
-                                             codes, stream);
+            e = launch_batch_backward<T, T>((const T *)path, (const T *)sig, (const T *)grad_sig, ginc, shape, plan, codes,
+                                            stream);
             profile_bracket(false, stream);
             if (e != hipSuccess) return launch_failed(e, "backward launch");
         }
     }
-    e = launch_increments_to_path<T>(ginc, (T *)grad_path, B, L, d, stream);
+    e = launch_increments_to_path<T, T>(ginc, (T *)grad_path, B, L, d, stream);
     if (e != hipSuccess) return launch_failed(e, "path-gradient launch");
     return PATHSIG_OK;
 }
@@ -437,7 +460,10 @@ size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d
     if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
     const DenseChoice dc =
         dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
-    return align_up((size_t)(B * (L - 1) * d) * elem_size(dtype)) + (dc.usable ? dc.backward_workspace : 0) + 256;
+    const bool words_kernel = !dc.usable && !batch_backward_usable(elem_size(dtype), B, d, W > 0 ? W : 1);
+    const bool batch_wide = !dc.usable && !words_kernel && batch_wide_sums(elem_size(dtype), plan);
+    return inc_buffer_bytes(elem_size(dtype), B, L, d, words_kernel || batch_wide) +
+           (dc.usable ? dc.backward_workspace : 0) + 256;
 }
 
 int pathsig_sig_backward(const void *path, const void *sig, const void *grad_sig, void *grad_path, int dtype,

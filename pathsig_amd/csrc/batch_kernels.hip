@@ -41,9 +41,9 @@ __device__ __forceinline__ int find_level_descending(const LevelPlan &plan, int6
     return deg;
 }
 
-template <typename T, int DEG, int G>
+template <typename T, int DEG, int G, typename ACC>
 __device__ void batch_backward_body(const T *__restrict__ path, const T *__restrict__ sig,
-                                    const T *__restrict__ grad_sig, T *__restrict__ grad_inc, const SigShape &shape,
+                                    const T *__restrict__ grad_sig, ACC *__restrict__ grad_inc, const SigShape &shape,
                                     const LevelPlan &plan, const int64_t *__restrict__ codes, int64_t blk_in_level,
                                     int tile, T *sdx, T *slabs) {
     constexpr int WPL = batch_words(DEG);
@@ -208,7 +208,7 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
         for (int pp = 0; pp < kPaths; ++pp) {
             const int q = wave + pp * kBatchWaves;
             const bool ok = b0 + q < shape.B;
-            T *gq = grad_inc + ((ok ? b0 + q : 0) * (shape.L - 1) + span.start + t0) * d;
+            ACC *gq = grad_inc + ((ok ? b0 + q : 0) * (shape.L - 1) + span.start + t0) * d;
             for (int j = lane; j < nt * d; j += kWave) {
                 // all reads first, so their latencies overlap
                 T *cell = slabs + j * kStride + q;
@@ -224,18 +224,18 @@ __device__ void batch_backward_body(const T *__restrict__ path, const T *__restr
                 T v = T(0);
 #pragma unroll
                 for (int i = 0; i < kBatchWaves * kSlots; ++i) v += part[i];
-                if (ok && v != T(0)) atomicAdd(&gq[j], v);
+                if (ok && v != T(0)) atomicAdd(&gq[j], (ACC)v);
             }
         }
         if (ti > 0) commit(tile_steps(ti - 1));
     }
 }
 
-template <typename T, int MAXDEG, int G>
+template <typename T, int MAXDEG, int G, typename ACC>
 __global__ void __launch_bounds__(kBatchBlock) batch_backward_kernel(const T *__restrict__ path,
                                                                      const T *__restrict__ sig,
                                                                      const T *__restrict__ grad_sig,
-                                                                     T *__restrict__ grad_inc, SigShape shape,
+                                                                     ACC *__restrict__ grad_inc, SigShape shape,
                                                                      LevelPlan plan, const int64_t *__restrict__ codes,
                                                                      int tile) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -248,7 +248,7 @@ __global__ void __launch_bounds__(kBatchBlock) batch_backward_kernel(const T *__
 #define PSIG_CASE(N)                                                                                                \
     case N:                                                                                                         \
         if constexpr (N <= MAXDEG)                                                                                  \
-            batch_backward_body<T, N, G>(path, sig, grad_sig, grad_inc, shape, plan, codes, bl, tile, sdx, slabs);   \
+            batch_backward_body<T, N, G, ACC>(path, sig, grad_sig, grad_inc, shape, plan, codes, bl, tile, sdx, slabs); \
         break;
         PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
         PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
@@ -285,8 +285,8 @@ bool batch_backward_usable(size_t elem, int64_t B, int64_t d, int64_t W) {
     return groups * W <= 65535;
 }
 
-template <typename T>
-hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
+template <typename T, typename ACC>
+hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig, ACC *grad_inc, const SigShape &shape,
                                  const LevelPlan &plan_in, const int64_t *codes, hipStream_t stream) {
     const int G = batch_group<T>(shape.B);
     LevelPlan plan = plan_in;
@@ -313,10 +313,10 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
 #define PSIG_LAUNCH(MAXDEG, GG)                                                                                    \
     do {                                                                                                           \
         if (lds > 64 * 1024)                                                                                       \
-            attr = hipFuncSetAttribute((const void *)batch_backward_kernel<T, MAXDEG, GG>,                         \
+            attr = hipFuncSetAttribute((const void *)batch_backward_kernel<T, MAXDEG, GG, ACC>,                    \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                      \
         if (attr != hipSuccess) return attr;                                                                       \
-        hipLaunchKernelGGL((batch_backward_kernel<T, MAXDEG, GG>), grid, dim3(kBatchBlock), lds, stream, path,     \
+        hipLaunchKernelGGL((batch_backward_kernel<T, MAXDEG, GG, ACC>), grid, dim3(kBatchBlock), lds, stream, path, \
                            sig, grad_sig, grad_inc, shape, plan, codes, (int)tile);                                \
     } while (0)
 #define PSIG_PICK(GG)                          \
@@ -335,9 +335,19 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
     return hipGetLastError();
 }
 
-template hipError_t launch_batch_backward<float>(const float *, const float *, const float *, float *,
-                                                 const SigShape &, const LevelPlan &, const int64_t *, hipStream_t);
-template hipError_t launch_batch_backward<double>(const double *, const double *, const double *, double *,
-                                                  const SigShape &, const LevelPlan &, const int64_t *, hipStream_t);
+// The flush adds one term per block (a slice of the words) to every (path, increment, letter) cell.  On dense levels of
+// a million words and more an fp32 cell collects tens of thousands of terms of mixed sign; such calls keep the
+// per-increment sums in fp64.
+bool batch_wide_sums(size_t elem, const LevelPlan &plan) { return elem == 4 && plan.sig_size >= 65536; }
+
+template hipError_t launch_batch_backward<float, float>(const float *, const float *, const float *, float *,
+                                                        const SigShape &, const LevelPlan &, const int64_t *,
+                                                        hipStream_t);
+template hipError_t launch_batch_backward<float, double>(const float *, const float *, const float *, double *,
+                                                         const SigShape &, const LevelPlan &, const int64_t *,
+                                                         hipStream_t);
+template hipError_t launch_batch_backward<double, double>(const double *, const double *, const double *, double *,
+                                                          const SigShape &, const LevelPlan &, const int64_t *,
+                                                          hipStream_t);
 
 }  // namespace psig

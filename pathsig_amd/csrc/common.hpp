@@ -113,14 +113,17 @@ struct Recip {
 template <typename T>
 hipError_t launch_words_forward(const T *path, T *sig, const SigShape &shape, const LevelPlan &plan,
                                 const int64_t *codes, hipStream_t stream);
+// (its per-increment sums are fp64 whatever T is: one term per block of words and cell)
 template <typename T>
-hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
-                                 const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
+hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, double *grad_inc,
+                                 const SigShape &shape, const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 // backward with lanes on paths (batch_kernels.hip): same contract as launch_words_backward; usable for
 // batches of at least a dozen paths of moderate dimension
 bool batch_backward_usable(size_t elem, int64_t B, int64_t d, int64_t W);
-template <typename T>
-hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
+// (ACC: type of the per-increment sums, T or, for fp32 calls where batch_wide_sums says so, double)
+bool batch_wide_sums(size_t elem, const LevelPlan &plan);
+template <typename T, typename ACC>
+hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig, ACC *grad_inc, const SigShape &shape,
                                  const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream);
@@ -131,8 +134,8 @@ hipError_t launch_gather_columns(const T *dense, T *out, const LevelPlan &plan, 
 template <typename T>
 hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan, int64_t d, const int64_t *codes,
                                   int64_t rows, hipStream_t stream);
-template <typename T>
-hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
+template <typename TI, typename T>
+hipError_t launch_increments_to_path(const TI *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
                                      hipStream_t stream);
 // sig -> logsig and the cache its adjoint reads; `powers`, when not null, also receives the power cache of the
 // reference (it may be the same buffer as `cache`, which it then replaces)

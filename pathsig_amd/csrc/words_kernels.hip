@@ -104,7 +104,7 @@ constexpr int kSortedMax = 64;
 
 template <typename T, int DEG>
 __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
-                              T *__restrict__ grad_inc, const SigShape &shape, const LevelPlan &plan,
+                              double *__restrict__ grad_inc, const SigShape &shape, const LevelPlan &plan,
                               const int64_t *__restrict__ codes, int64_t row, int64_t blk_in_level, int tile, T *sdx,
                               T *sacc, T *sval, int *sorder, int *scnt) {
     const int lane = threadIdx.x;
@@ -160,7 +160,7 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
     const int64_t b = row / shape.W, w = row - b * shape.W;
     const WindowSpan span = window_span(shape, w);
     const T *x = path + (b * shape.L + span.start) * d;
-    T *ginc = grad_inc + (b * (shape.L - 1) + span.start) * d;
+    double *ginc = grad_inc + (b * (shape.L - 1) + span.start) * d;
     const T *srow = sig + row * plan.sig_size;
 
     // chain of prefix values at the right end of the window (levels < DEG)
@@ -271,7 +271,9 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
         __syncthreads();
         for (int64_t idx = lane; idx < (int64_t)nt * d; idx += kBwdBlock) {
             const T v = sacc[idx];
-            if (v != T(0)) atomicAdd(&ginc[t0 * d + idx], v);
+            // one term per block of words: summed in fp64, because a dense level of millions of words adds tens of
+            // thousands of them to one cell (fp32 there: 2e-5 to 3e-5 of the largest gradient lost at (8,8))
+            if (v != T(0)) atomicAdd(&ginc[t0 * d + idx], (double)v);
         }
     }
 }
@@ -281,7 +283,7 @@ __device__ void backward_body(const T *__restrict__ path, const T *__restrict__ 
 template <typename T, int MAXDEG>
 __global__ void __launch_bounds__(kBwdBlock) words_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig,
                                                                    const T *__restrict__ grad_sig,
-                                                                   T *__restrict__ grad_inc, SigShape shape,
+                                                                   double *__restrict__ grad_inc, SigShape shape,
                                                                    LevelPlan plan, const int64_t *__restrict__ codes,
                                                                    int tile) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -317,8 +319,9 @@ __global__ void fill_zero_kernel(T *__restrict__ ptr, int64_t n) {
 
 // dL/dx[t] = dL/d(dx[t-1]) - dL/d(dx[t]) with one-sided ends
 // (reference: src/pathsig/backward/sig_backward_kernels.cu:347-377; 64-bit indices here)
-template <typename T>
-__global__ void increments_to_path_kernel(const T *__restrict__ ginc, T *__restrict__ gpath, int64_t B, int64_t L,
+// (TI: type of the per-increment sums, fp64 behind the word-per-lane backward)
+template <typename TI, typename T>
+__global__ void increments_to_path_kernel(const TI *__restrict__ ginc, T *__restrict__ gpath, int64_t B, int64_t L,
                                           int64_t d) {
     const int64_t total = B * L * d;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -327,10 +330,10 @@ __global__ void increments_to_path_kernel(const T *__restrict__ ginc, T *__restr
         const int64_t rem = i - b * L * d;
         const int64_t t = rem / d;
         const int64_t a = rem - t * d;
-        const T *g = ginc + b * (L - 1) * d + a;
-        const T left = t > 0 ? g[(t - 1) * d] : T(0);
-        const T right = t < L - 1 ? g[t * d] : T(0);
-        gpath[i] = left - right;
+        const TI *g = ginc + b * (L - 1) * d + a;
+        const TI left = t > 0 ? g[(t - 1) * d] : TI(0);
+        const TI right = t < L - 1 ? g[t * d] : TI(0);
+        gpath[i] = (T)(left - right);
     }
 }
 
@@ -423,7 +426,7 @@ hipError_t launch_words_forward(const T *path, T *sig, const SigShape &shape, co
 }
 
 template <typename T>
-hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, const SigShape &shape,
+hipError_t launch_words_backward(const T *path, const T *sig, const T *grad_sig, double *grad_inc, const SigShape &shape,
                                  const LevelPlan &plan_in, const int64_t *codes, hipStream_t stream) {
     // same levels, blocks of one wave
     LevelPlan plan = plan_in;
@@ -461,14 +464,14 @@ hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <typename T>
-hipError_t launch_increments_to_path(const T *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
+template <typename TI, typename T>
+hipError_t launch_increments_to_path(const TI *grad_inc, T *grad_path, int64_t B, int64_t L, int64_t d,
                                      hipStream_t stream) {
     const int64_t n = B * L * d;
     if (n <= 0) return hipSuccess;
     int64_t blocks = (n + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(increments_to_path_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_inc, grad_path,
+    hipLaunchKernelGGL((increments_to_path_kernel<TI, T>), dim3((unsigned)blocks), dim3(256), 0, stream, grad_inc, grad_path,
                        B, L, d);
     return hipGetLastError();
 }
@@ -504,12 +507,14 @@ hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan
                                                   int64_t, hipStream_t);                                            \
     template hipError_t launch_words_forward<T>(const T *, T *, const SigShape &, const LevelPlan &, const int64_t *, \
                                                 hipStream_t);                                                       \
-    template hipError_t launch_words_backward<T>(const T *, const T *, const T *, T *, const SigShape &,            \
+    template hipError_t launch_words_backward<T>(const T *, const T *, const T *, double *, const SigShape &,       \
                                                  const LevelPlan &, const int64_t *, hipStream_t);                  \
     template hipError_t launch_fill_zero<T>(T *, int64_t, hipStream_t);                                             \
-    template hipError_t launch_increments_to_path<T>(const T *, T *, int64_t, int64_t, int64_t, hipStream_t);
+    template hipError_t launch_increments_to_path<T, T>(const T *, T *, int64_t, int64_t, int64_t, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE
+template hipError_t launch_increments_to_path<double, float>(const double *, float *, int64_t, int64_t, int64_t,
+                                                               hipStream_t);
 
 }  // namespace psig
