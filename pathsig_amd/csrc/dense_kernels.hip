@@ -1205,6 +1205,10 @@ __device__ __forceinline__ void dense_backward_body(
     // registers are plentiful; otherwise the letters are compared every time)
     constexpr bool kOneHot = sizeof(T) == 4 && P * D <= 24;
     T onehot[kOneHot ? P : 1][kOneHot ? D : 1];
+    // Wide alphabets compare every letter with the prefix letters to route the chain's terms (P * D selects and
+    // adds per increment).  The last prefix letter is different in every lane of a row of sixteen, so its term
+    // is added to the row's cell of that letter in LDS instead, after the pass that writes the cells.
+    constexpr bool kLastDirect = !kOneHot && !BS::kChainCells && D >= 16 && kParts == 4;
     if constexpr (kOneHot) {
 #pragma unroll
         for (int j = 0; j < P; ++j)
@@ -1257,7 +1261,7 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int q = 1; q < KS; ++q) v = fmad<T>(gdxk[q][k], rcp<T>(q + 1), v);
 #pragma unroll
-                for (int j = 0; j < P; ++j) {
+                for (int j = 0; j < (kLastDirect ? P - 1 : P); ++j) {
                     if constexpr (kOneHot) v = fmad<T>(onehot[j][k], gpre[j], v);
                     else if constexpr (!BS::kChainCells) v += (u[j] == k) ? gpre[j] : T(0);
                 }
@@ -1285,6 +1289,11 @@ __device__ __forceinline__ void dense_backward_body(
                     const T r = row_totals<T, DP>(padded, lane);
                     const int letter = base + row_letter<DP>(lane);
                     if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
+                }
+                if constexpr (kLastDirect) {
+                    // the term of the last prefix letter goes straight to its cell: the sixteen lanes of a row hold
+                    // consecutive prefixes, so with sixteen letters or more their last letters differ
+                    if (active) sg[wave * 4 + (lane >> 4)][tt * D + u[P - 1]] += gpre[P - 1];
                 }
                 if constexpr (G::kSplit) {
                     // The lane's own children carry the letters a0 .. a0 + K - 1, the same for the whole wave.  Their
