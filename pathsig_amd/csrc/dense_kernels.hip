@@ -1209,6 +1209,27 @@ __device__ __forceinline__ void dense_backward_body(
     // adds per increment).  The last prefix letter is different in every lane of a row of sixteen, so its term
     // is added to the row's cell of that letter in LDS instead, after the pass that writes the cells.
     constexpr bool kLastDirect = !kOneHot && !BS::kChainCells && D >= 16 && kParts == 4;
+    // The earlier prefix letters take at most two values within such a row (sixteen consecutive prefixes cross at
+    // most one multiple of D, D^2, ..): the letter of the row's first lane and that of its last.  Their terms are
+    // summed over the row in those two groups and added to the two cells by the row's first lane.
+    constexpr int kRowLetters = kLastDirect ? P - 1 : 0;
+    int ua[kRowLetters > 0 ? kRowLetters : 1], ub[kRowLetters > 0 ? kRowLetters : 1];
+    bool with_first[kRowLetters > 0 ? kRowLetters : 1];
+    bool row_live = false;
+    if constexpr (kRowLetters > 0) {
+        const int first = pu - (lane & 15);
+        row_live = first < G::kPrefixes;
+        const int last = first + 15 < G::kPrefixes ? first + 15 : G::kPrefixes - 1;
+        int uf[P], ul[P];
+        prefix_letters<D, P>(row_live ? first : 0, uf);
+        prefix_letters<D, P>(row_live ? last : 0, ul);
+#pragma unroll
+        for (int j = 0; j < kRowLetters; ++j) {
+            ua[j] = uf[j];
+            ub[j] = ul[j];
+            with_first[j] = u[j] == uf[j];
+        }
+    }
     if constexpr (kOneHot) {
 #pragma unroll
         for (int j = 0; j < P; ++j)
@@ -1261,7 +1282,7 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int q = 1; q < KS; ++q) v = fmad<T>(gdxk[q][k], rcp<T>(q + 1), v);
 #pragma unroll
-                for (int j = 0; j < (kLastDirect ? P - 1 : P); ++j) {
+                for (int j = 0; j < (kLastDirect ? 0 : P); ++j) {
                     if constexpr (kOneHot) v = fmad<T>(onehot[j][k], gpre[j], v);
                     else if constexpr (!BS::kChainCells) v += (u[j] == k) ? gpre[j] : T(0);
                 }
@@ -1294,6 +1315,17 @@ __device__ __forceinline__ void dense_backward_body(
                     // the term of the last prefix letter goes straight to its cell: the sixteen lanes of a row hold
                     // consecutive prefixes, so with sixteen letters or more their last letters differ
                     if (active) sg[wave * 4 + (lane >> 4)][tt * D + u[P - 1]] += gpre[P - 1];
+#pragma unroll
+                    for (int j = 0; j < kRowLetters; ++j) {
+                        const T mine = with_first[j] ? gpre[j] : T(0);
+                        const T sum_first = row_total(mine);
+                        const T sum_last = row_total(gpre[j] - mine);
+                        if ((lane & 15) == 0 && row_live) {
+                            T *cells_of_step = &sg[wave * 4 + (lane >> 4)][tt * D];
+                            cells_of_step[ua[j]] += sum_first;
+                            if (ub[j] != ua[j]) cells_of_step[ub[j]] += sum_last;
+                        }
+                    }
                 }
                 if constexpr (G::kSplit) {
                     // The lane's own children carry the letters a0 .. a0 + K - 1, the same for the whole wave.  Their
