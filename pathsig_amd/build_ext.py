@@ -40,10 +40,10 @@ HIPCC_FLAGS = [
 ]
 
 
-def _compile(unit, verbose: bool) -> pathlib.Path:
+def _compile(unit, verbose: bool, obj_dir: pathlib.Path, defines) -> pathlib.Path:
     src, obj_name, extra = unit
-    obj = CSRC / obj_name
-    cmd = ["hipcc", *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
+    obj = obj_dir / obj_name
+    cmd = ["hipcc", *HIPCC_FLAGS, *defines, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -57,17 +57,26 @@ def _compile(unit, verbose: bool) -> pathlib.Path:
     return obj
 
 
-def build(verbose: bool = False, jobs: int = 8) -> pathlib.Path:
+def build(verbose: bool = False, jobs: int = 8, only=None, out_dir: pathlib.Path | None = None) -> pathlib.Path:
+    """only: iterable of (d, depth) pairs; the register-tiled kernels are then compiled for these shapes alone (a
+    small library that builds in a minute; every other shape runs on the per-word kernels).
+    out_dir: where the objects and the library go (default: beside the sources / in the package)."""
+    defines = []
+    if only:
+        defines = ["-DPSIG_ONLY=" + ",".join("{%d,%d}" % (int(d), int(n)) for d, n in only)]
+    lib = LIB if out_dir is None else pathlib.Path(out_dir) / LIB.name
+    obj_dir = CSRC if out_dir is None else pathlib.Path(out_dir) / "obj"
+    obj_dir.mkdir(parents=True, exist_ok=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda u: _compile(u, verbose), UNITS))
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
+        objs = list(pool.map(lambda u: _compile(u, verbose, obj_dir, defines), UNITS))
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib), *map(str, objs)]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return LIB
+    return lib
 
 
-def build_torch_ops(verbose: bool = False) -> pathlib.Path:
+def build_torch_ops(verbose: bool = False, out_dir: pathlib.Path | None = None) -> pathlib.Path:
     """C++ registration of the operators with the torch dispatcher (host code only; needs libpathsig_hip.so)."""
     import torch
     from torch.utils import cpp_extension
@@ -76,20 +85,30 @@ def build_torch_ops(verbose: bool = False) -> pathlib.Path:
         raise RuntimeError("the operator library needs a ROCm build of PyTorch")
     includes = [f"-I{p}" for p in cpp_extension.include_paths()] + ["-I/opt/rocm/include", f"-I{INCLUDE}"]
     lib_dirs = cpp_extension.library_paths()
+    pkg = PKG if out_dir is None else pathlib.Path(out_dir)
+    torch_lib = pkg / TORCH_LIB.name
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", *includes,
-           str(CSRC / "torch_ops.cpp"), "-o", str(TORCH_LIB),
+           str(CSRC / "torch_ops.cpp"), "-o", str(torch_lib),
            *[f"-L{d}" for d in lib_dirs], "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
-           f"-L{PKG}", "-lpathsig_hip", "-Wl,-rpath,$ORIGIN", *[f"-Wl,-rpath,{d}" for d in lib_dirs]]
+           f"-L{pkg}", "-lpathsig_hip", "-Wl,-rpath,$ORIGIN", *[f"-Wl,-rpath,{d}" for d in lib_dirs]]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
         raise RuntimeError("g++ failed on torch_ops.cpp")
-    return TORCH_LIB
+    return torch_lib
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
-    print(build_torch_ops(verbose=True))
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--only", default=None, metavar="DxN[,DxN...]",
+                    help="compile the register-tiled kernels for these (d, depth) shapes only, e.g. 4x6,8x4")
+    ap.add_argument("--out-dir", default=None, help="directory for the objects and the two libraries")
+    opts = ap.parse_args()
+    shapes = [tuple(int(v) for v in item.split("x")) for item in opts.only.split(",")] if opts.only else None
+    print(build(verbose=True, only=shapes, out_dir=opts.out_dir))
+    print(build_torch_ops(verbose=True, out_dir=opts.out_dir))

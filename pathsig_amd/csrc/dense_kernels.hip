@@ -1584,7 +1584,26 @@ const int *stage_letter_bounds(const DenseChoice &dc, const int64_t *top_codes, 
 
 #endif
 
-#define PSIG_INFO(I, D, N, P, PC, PS) variant_info<D, N, P, PS>(),
+// A reduced library: -DPSIG_ONLY="{4,6},{8,4}" compiles the register-tiled kernels of the listed (d, depth) pairs
+// only; every other shape then runs on the per-word kernels.  (The full table takes minutes to compile.)
+#ifdef PSIG_ONLY
+constexpr int kOnlyShapes[][2] = {PSIG_ONLY};
+constexpr bool shape_enabled(int d, int depth) {
+    for (const auto &s : kOnlyShapes)
+        if (s[0] == d && s[1] == depth) return true;
+    return false;
+}
+#else
+constexpr bool shape_enabled(int, int) { return true; }
+#endif
+
+template <int D, int N, int P, int PS>
+constexpr VariantInfo variant_info_if_enabled() {
+    if constexpr (shape_enabled(D, N)) return variant_info<D, N, P, PS>();
+    else return VariantInfo{-1, -1, 0, 0, 0, 0, false, {false, false}, false};
+}
+
+#define PSIG_INFO(I, D, N, P, PC, PS) variant_info_if_enabled<D, N, P, PS>(),
 constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
 #undef PSIG_INFO
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -1975,12 +1994,12 @@ static_assert(PSIG_GROUP < kDenseGroups, "group index out of range");
 
 #define PSIG_CASE_FWD(I, D, N, P, PC, PS)                                                                         \
     case I:                                                                                                       \
-        if constexpr (I % kDenseGroups == PSIG_GROUP)                                                             \
+        if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                      \
             return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace, stream); \
         break;
 #define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
     case I:                                                                                                        \
-        if constexpr (I % kDenseGroups == PSIG_GROUP)                                                              \
+        if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                       \
             return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape,       \
                                                 dc.bwd_chunks, bounds, kept, workspace, stream);                   \
         break;

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
-from .ops import compute_signature, sig_to_logsig
+from .ops import _logsig_of, compute_signature
 
 _DEVICE = "cuda"
 
@@ -102,7 +102,7 @@ class LogSignature(nn.Module):
         top_words = self._top_words
         sig = compute_signature(path, self.depth, self.alternative_projection, top_words, sizes, self.use_windows,
                                 self._windows)
-        logsig, _ = sig_to_logsig(sig, self.depth, d, self.alternative_projection, top_words, sizes)
+        logsig = _logsig_of(sig, self.depth, d, self.alternative_projection, top_words, sizes)
         if not self.alternative_projection:
             return logsig
         return logsig.index_select(dim=-1, index=self._indices_from_sig.to(logsig.device))

@@ -65,15 +65,25 @@ def compute_signature(path: Tensor, depth: int, alternative_projection: bool, en
 
 def sig_to_logsig(signature: Tensor, depth: int, d: int, alternative_projection: bool, encoded_words: Tensor,
                   level_sizes: list[int]) -> tuple[Tensor, Tensor]:
-    """Signature in the hybrid layout -> (log-signature, cache).
+    """Signature in the hybrid layout -> (log-signature, P_arr).
 
-    Without a gradient the cache is the power cache of the reference; when a gradient will be asked for it is the
-    cache the adjoint reads (powers of the log-signature), so the backward need not rebuild it."""
-    if torch.is_grad_enabled() and signature.requires_grad and not os.environ.get("PATHSIG_NO_KEEP"):
-        return torch.ops.pathsig.sig_to_logsig_keep.default(
-            signature, depth, d, alternative_projection, encoded_words, level_sizes)
+    The second output is the power cache of the reference (`src/pathsig/ops.py:87-98`, layout of
+    `sig_kernels.cu:184,215-216`), with or without a gradient: a caller may read it or hand it to
+    `logsig_backward`."""
     return torch.ops.pathsig.sig_to_logsig.default(
         signature, depth, d, alternative_projection, encoded_words, level_sizes)
+
+
+def _logsig_of(signature: Tensor, depth: int, d: int, alternative_projection: bool, encoded_words: Tensor,
+               level_sizes: list[int]) -> Tensor:
+    """Log-signature alone, for the `LogSignature` module, which never shows the cache to its caller: when a
+    gradient will be asked for, the forward keeps the cache its own adjoint reads (powers of the log-signature)
+    in place of the reference's power cache, so the backward need not rebuild it."""
+    if torch.is_grad_enabled() and signature.requires_grad and not os.environ.get("PATHSIG_NO_KEEP"):
+        return torch.ops.pathsig.sig_to_logsig_keep.default(
+            signature, depth, d, alternative_projection, encoded_words, level_sizes)[0]
+    return torch.ops.pathsig.sig_to_logsig.default(
+        signature, depth, d, alternative_projection, encoded_words, level_sizes)[0]
 
 
 def signature_backward(path: Tensor, signature: Tensor, grad_signature: Tensor, depth: int,

@@ -313,6 +313,29 @@ def test_sig_to_logsig_cache_layout(ps):
     assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
 
 
+def test_public_sig_to_logsig_returns_the_power_cache_with_a_gradient_too(ps):
+    """`ops.sig_to_logsig` (`src/pathsig/ops.py:87-98`) returns the reference's P_arr whether or not its input
+    asks for a gradient, and the gradient through it agrees with the checker's adjoint."""
+    from pathsig_amd import ops
+    d, depth, B = 3, 4, 2
+    top = [5, 80, 17, 17, 2]
+    path = brownian_path(B, 9, d, seed=45)
+    cols = TO.hybrid_columns(d, depth, len(top), top)
+    hyb = TO.signature(path, depth)[:, cols]
+    want_log, want_P = TO.sig_to_logsig(hyb, depth, d, len(top), top)
+    sizes = [0] + [d ** k for k in range(1, depth)] + [len(top)]
+    words = torch.tensor(top, dtype=torch.int64, device=DEV)
+    sg = hyb.to(DEV).requires_grad_(True)
+    logsig, P = ops.sig_to_logsig(sg, depth, d, True, words, sizes)
+    assert rel_err(logsig, want_log) < 1e-12
+    assert rel_err(P, want_P) < 1e-12
+    g = randn(tuple(hyb.shape), seed=46)
+    (got,) = torch.autograd.grad(logsig, sg, g.to(DEV))
+    assert rel_err(got, TO.logsig_vjp(hyb, g, depth, d, len(top), top)) < 1e-12
+    again = ops.logsig_backward(sg.detach(), P.detach(), g.to(DEV), depth, True, words, sizes)
+    assert rel_err(again, got) < 1e-12
+
+
 def test_sig_to_logsig_keep_cache(ps):
     """The keeping forward returns the same log-signature and, as its cache, the tensor powers of that
     log-signature for the words below the top level (entry k - 1 of a word's row: its coefficient in L^(x)k;
