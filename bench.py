@@ -29,12 +29,16 @@ import time
 import torch
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}
-# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counters scaled on a
-# copy of known size (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00).  Summaries and commands:
-# profiles/dense_backward_kernel_c2.md, profiles/dense_kernels_c3_c5.md, profiles/batch_backward_kernel_c4.md.
-# c2, c4, c5: counters of the kernels as they are in this tree; c3: its kernel has not changed since its counters
-# were taken.  c4 counts the float atomics of the slab flush as written bytes (268 MB of the 377).
-TRAFFIC_BYTES = {("c2", "f32"): 50.0e6, ("c3", "f32"): 189.7e6, ("c4", "f32"): 377.4e6, ("c5", "f32"): 60.2e6}
+# HBM bytes per launch of the dominant kernel, keyed by workload: rocprofv3 FETCH_SIZE + WRITE_SIZE counters scaled
+# on a copy of known size (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00).  These are figures from the committed counter
+# summaries, not measured in this run; `source` names the summary.  c4 counts the float atomics of the slab flush as
+# written bytes (268 MB of the 377).
+TRAFFIC = {
+    ("c2", "f32"): {"bytes": 50.0e6, "source": "profiles/dense_backward_kernel_c2.md"},
+    ("c3", "f32"): {"bytes": 189.7e6, "source": "profiles/dense_kernels_c3_c5.md"},
+    ("c4", "f32"): {"bytes": 377.4e6, "source": "profiles/batch_backward_kernel_c4.md"},
+    ("c5", "f32"): {"bytes": 60.2e6, "source": "profiles/dense_kernels_c3_c5.md"},
+}
 
 
 # ------------------------------------------------------------------------------------------------
@@ -216,52 +220,11 @@ def cpu_baseline(wl, dtype, budget_s=20.0):
                       f"{'fwd+bwd' if cfg['backward'] else 'fwd'}, torch level-tensor checker, median of {max(reps, 1)}"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=300)
-    ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--settle-ms", type=float, default=1500.0,
-                    help="before the W warm-up steps, run untimed steps for this long so that the device has left "
-                         "its idle power state (its shader clock idles near 100 MHz and takes far longer than W short "
-                         "steps to reach 2.4 GHz); 0 switches it off")
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--shape", default=None, metavar="D,N[,B[,L]]",
-                    help="instead of a named configuration: dense signature of depth N in D dimensions, forward + "
-                         "backward, B paths (default 128) of L points (default 512); the tables of per-shape timings "
-                         "are made with this")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true",
-                    help="skip the extra leg that captures one step in a HIP graph and times replays of it "
-                         "(reported beside the eager figure as graph_replay; `value` is always the eager one)")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also copy one 256 MiB buffer once (untimed), as the known-size kernel that scales "
-                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
-                 "(paths are independent, so more GPUs would simply split the batch).")
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU")
-
-    if args.copy_calibration:
-        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    dtype = torch.float32 if args.dtype == "f32" else torch.float64
-    if args.shape:
-        parts = [int(v) for v in args.shape.split(",")]
-        d, depth = parts[0], parts[1]
-        B = parts[2] if len(parts) > 2 else 128
-        L = parts[3] if len(parts) > 3 else 512
-        args.config = "shape"
-        CONFIGS["shape"] = dict(op="sig", B=B, L=L, d=d, depth=depth, backward=True,
-                                desc=f"signature depth {depth} fwd+bwd, B={B} L={L} d={d}")
-    index = int(args.config[1]) if args.config != "shape" else 9
-    wl = make_workload(args.config, dtype, index)
+def run_config(name, dtype_name, args, with_graph, with_cpu, settle_ms):
+    """Times one workload and returns its result dictionary (the JSON line of a run on that workload)."""
+    dtype = torch.float32 if dtype_name == "f32" else torch.float64
+    index = int(name[1]) if name != "shape" else 9
+    wl = make_workload(name, dtype, index)
     cfg, mod, x, G = wl["cfg"], wl["mod"], wl["x"], wl["G"]
     B = cfg["B"]
 
@@ -279,7 +242,7 @@ def main():
         torch.autograd.grad(out, xg, G)
 
     # the device idles at a low shader clock: keep it busy until the clock has settled (untimed)
-    t_end = time.perf_counter() + args.settle_ms * 1e-3
+    t_end = time.perf_counter() + settle_ms * 1e-3
     while time.perf_counter() < t_end:
         for _ in range(20):
             step()
@@ -300,22 +263,22 @@ def main():
     ms_per_step = 1e3 * elapsed / args.steps
 
     fwd_mean, fwd_med = time_events(fwd_only, args.steps, 3)
-    peak = PEAK_TFLOPS[args.dtype]
+    peak = PEAK_TFLOPS[dtype_name]
     result = {
-        "metric": metric_name(args.config, cfg, args.dtype),
+        "metric": metric_name(name, cfg, dtype_name),
         "value": B / (ms_per_step * 1e-3),
         "unit": "paths/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "settle_ms": args.settle_ms,
+        "settle_ms": settle_ms,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": args.dtype,
+        "dtype": dtype_name,
         "data": "synthetic",
-        "config": {"workload": f"{args.config}: {cfg['desc']}, {args.dtype}",
+        "config": {"workload": f"{name}: {cfg['desc']}, {dtype_name}",
                    "step": "forward + backward" if cfg["backward"] else "forward",
                    "launch": "eager",
                    "out_shape": list(wl["out_shape"]), "horner_nodes_per_increment": wl["nodes"]},
@@ -335,7 +298,6 @@ def main():
                 args_b = (x, sig, G, mod.depth, mod.alternative_projection, mod._encoded_words, mod._level_sizes,
                           mod.use_windows, mod._windows)
             else:
-                d = cfg["d"]
                 sizes = mod._ext_level_sizes
                 sig = torch.ops.pathsig.compute_signature(x, mod.depth, True, mod._top_words, sizes, mod.use_windows,
                                                           mod._windows)
@@ -361,16 +323,19 @@ def main():
         if sweep:
             sweep_ms = sum(sweep) / len(sweep)
             ach_k = 3.0 * wl["fwd_flops"] / (sweep_ms * 1e-3) / 1e12
+            kernel = ("dense_backward_kernel (reverse sweep)" if cfg.get("words") is None
+                      else "batch_backward_kernel (reverse sweep, lanes on paths)")
+            traffic = TRAFFIC.get((name, dtype_name))
             result["roofline"] = {"bound": "valu", "achieved": ach_k, "peak": peak, "unit": "TFLOP/s",
-                                  "frac": ach_k / peak, "traffic": TRAFFIC_BYTES.get((args.config, args.dtype)),
-                                  "kernel": ("dense_backward_kernel (reverse sweep)" if cfg.get("words") is None
-                                             else "batch_backward_kernel (reverse sweep, lanes on paths)"),
-                                  "kernel_ms": sweep_ms}
+                                  "frac": ach_k / peak, "traffic": None if traffic is None else traffic["bytes"],
+                                  "kernel": kernel, "kernel_ms": sweep_ms}
+            if traffic is not None:
+                result["roofline"]["traffic_source"] = traffic["source"]
         else:
             result["roofline"] = dict(result["roofline_backward_call"])
     else:
         result["roofline"] = dict(result["roofline_forward"], kernel="signature forward call")
-    if not args.no_graph:
+    if with_graph:
         # the same step captured once in a HIP graph and replayed: what a caller gets who takes the Python and
         # launch overhead out of the loop (the library neither allocates nor synchronises, so it captures)
         try:
@@ -390,8 +355,78 @@ def main():
             del graph
         except Exception as exc:  # a capture failure must not cost the eager figures
             result["graph_replay"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
-    if not args.no_cpu:
+    if with_cpu:
         result["cpu_baseline"] = cpu_baseline(wl, dtype)
+    return result
+
+
+# the other workloads of the metric, timed in the same run as the headline one (same steps and warm-up)
+OTHER_WORKLOADS = (("c1", "f32"), ("c3", "f32"), ("c4", "f32"), ("c5", "f32"), ("c5", "f64"))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-ms", type=float, default=1500.0,
+                    help="before the W warm-up steps, run untimed steps for this long so that the device has left "
+                         "its idle power state (its shader clock idles near 100 MHz and takes far longer than W short "
+                         "steps to reach 2.4 GHz); 0 switches it off")
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--shape", default=None, metavar="D,N[,B[,L]]",
+                    help="instead of a named configuration: dense signature of depth N in D dimensions, forward + "
+                         "backward, B paths (default 128) of L points (default 512); the tables of per-shape timings "
+                         "are made with this")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the extra leg that captures one step in a HIP graph and times replays of it "
+                         "(reported beside the eager figure as graph_replay; `value` is always the eager one)")
+    ap.add_argument("--no-others", action="store_true",
+                    help="a run on the headline workload (the default) also times the other workloads of the metric "
+                         "(c1, c3, c4, c5 in fp32 and fp64) with the same steps and reports them under "
+                         "`other_configs`; this switches that off")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also copy one 256 MiB buffer once (untimed), as the known-size kernel that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
+                 "(paths are independent, so more GPUs would simply split the batch).")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.shape:
+        parts = [int(v) for v in args.shape.split(",")]
+        d, depth = parts[0], parts[1]
+        B = parts[2] if len(parts) > 2 else 128
+        L = parts[3] if len(parts) > 3 else 512
+        args.config = "shape"
+        CONFIGS["shape"] = dict(op="sig", B=B, L=L, d=d, depth=depth, backward=True,
+                                desc=f"signature depth {depth} fwd+bwd, B={B} L={L} d={d}")
+    result = run_config(args.config, args.dtype, args, not args.no_graph, not args.no_cpu, args.settle_ms)
+    if args.config == "c2" and args.dtype == "f32" and not args.no_others:
+        others = {}
+        for name, dtype_name in OTHER_WORKLOADS:
+            # (the device is busy already: a short settling phase is enough)
+            r = run_config(name, dtype_name, args, False, False, min(args.settle_ms, 300.0))
+            keep = {k: r[k] for k in ("value", "unit", "ms_per_step", "fwd_paths_per_s", "fwd_ms", "step_tflops",
+                                      "step_frac_of_peak", "dtype") if k in r}
+            keep["workload"] = r["config"]["workload"]
+            keep["step"] = r["config"]["step"]
+            if "bwd_ms" in r:
+                keep["bwd_ms"] = r["bwd_ms"]
+            keep["roofline"] = r["roofline"]
+            others[f"{name}_{dtype_name}"] = keep
+            torch.cuda.empty_cache()
+        result["other_configs"] = others
     print(json.dumps(result))
 
 

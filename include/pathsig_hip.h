@@ -92,9 +92,11 @@ int pathsig_sig_backward_noalloc(const void *path, const void *sig, const void *
 /*
  * The same pair with a hand-over from the forward to the backward of one call (no counterpart in the
  * reference, whose backward receives the path and the signature only and recomputes what it needs).
- * On long paths the register-tiled kernels cut every row into time chunks; the forward can write the
- * signature of each chunk below the top level into `chunks`, and a backward that is given the same buffer
- * skips the launch that would recompute them.  The per-word kernels hand over, in the same buffer, the
+ * On long paths the register-tiled kernels cut every row into time chunks; the backward starts every chunk
+ * from the signature of the row up to the chunk's right edge and from the signature of the rest of the row,
+ * both below the top level (products of the chunks' own signatures).  The forward can write those two
+ * arrays into `chunks`, and a backward that is given the same buffer skips the two launches that would
+ * recompute them.  The per-word kernels hand over, in the same buffer, the
  * prefix values of the words whose prefixes are not all part of the signature (the backward otherwise
  * rebuilds them with a forward sweep, as src/pathsig/backward/sig_backward_kernels.cu:134-157 does).
  * A word projection that is computed through a register-tiled shape which is swept in one piece (depth 2,

@@ -394,6 +394,7 @@ int pathsig_set_option(const char *name, int64_t value) {
         option_cells().embed_share.store(value, std::memory_order_relaxed);
     } else if (!strcmp(name, "tiled") && (value == 0 || value == 1)) {
         option_cells().tiled.store(value, std::memory_order_relaxed);
+
     } else {
         set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
         return PATHSIG_ERR_ARGUMENT;

@@ -17,8 +17,8 @@ struct DenseChoice {
     size_t dense_bytes;         // embed: bytes of one dense [rows, S] buffer
     size_t forward_workspace;   // bytes of scratch the forward needs (including the dense buffer)
     size_t backward_workspace;  // bytes of scratch the backward needs beyond the increment accumulator
-    size_t keep_bytes;          // bytes the forward can keep for the backward: chunk signatures, or (resweep) the
-                                // dense signature (0: none)
+    size_t keep_bytes;          // bytes the forward can keep for the backward: the prefix and suffix products of the
+                                // chunk signatures below the top level, or (resweep) the dense signature (0: none)
 };
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,
@@ -26,8 +26,9 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
 
 // `sig` / `grad_sig` are dense-layout rows; `workspace` is the part of the scratch after any dense buffer.
 // top_codes / top_count: the word list of the top level (device memory), read only when dc.bounded.
-// keep (optional, dc.keep_bytes bytes): receives the signatures of the time chunks below the top level; passing
-// the same buffer as `kept` to the backward of the same call saves it the launch that recomputes them.
+// keep (optional, dc.keep_bytes bytes): receives, per time chunk, the signature of the row up to the chunk's right
+// edge and that of the rest of the row, below the top level; passing the same buffer as `kept` to the backward of
+// the same call saves it the launches that recompute them.
 template <typename T>
 hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, const DenseChoice &dc,
                                 const int64_t *top_codes, int64_t top_count, T *keep, void *workspace,

@@ -23,6 +23,7 @@
 // gradient.  Adjoint values of the shared chain nodes stay lane-private partial sums (everything they
 // feed is linear in them), so the only cross-lane operation is the final sum of D numbers per step.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
@@ -1115,20 +1116,42 @@ __global__ void __launch_bounds__(kWave) chunk_level1_kernel(const T *__restrict
     }
 }
 
-// LDS layout of the reverse sweep.  Per-increment sums leave a wave as four row sums; the tile flush adds the
-// parts of all waves in a fixed order.  The tile is shortened until the parts fit 48 KB of LDS (128 KB for the
-// widest alphabets, whose parts of sixteen increments would not fit a CU at all).
+// LDS layout of the reverse sweep.  Per-increment sums leave a wave as four row sums (eight partial sums where the
+// slab below is used); the tile flush adds the parts of all waves in a fixed order.  The tile is shortened until
+// the parts fit 48 KB of LDS (128 KB for the widest alphabets, whose parts of sixteen increments would not fit a
+// CU at all).
+//
+// The slab.  Summing a lane's D per-increment terms over the lanes with DPP moves costs more than its dozen
+// instructions: a wave with DPP instructions (or lane reads, or lane permutes) in its stream is not overlapped
+// with the other wave of its SIMD any more.  Measured on MI355X with two resident waves per SIMD: 0.94 ns per
+// vector instruction for a long run of multiply-adds, 1.7 to 1.8 ns as soon as one instruction in sixty-four
+// is a DPP move, which is what one wave alone gets; LDS reads, writes and swizzles cost about three instruction
+// slots each and leave the overlap alone.  The loop of the depth-6 sweep over four letters: 1.39 ns per vector
+// instruction as compiled, 1.11 ns with its twelve DPP instructions replaced by plain ones.  So fp32 units of up
+// to four waves over at most fifteen letters take another way: every lane stores its D terms of an increment,
+// padded to kDP, into a slab of its wave (one or more 16-byte LDS stores), and once kSubTile increments have
+// gathered there the lanes read the slab back across the lanes, eight 16-byte reads each, and leave eight
+// partial sums per increment and letter in `sg`.
 template <typename T, int D, int N, int P>
 struct BackwardShape {
     using G = Geometry<D, N, P, sizeof(T)>;
     static constexpr int KS = N - P;
-    static constexpr int kParts = 4;
-    static constexpr int kRowBytes = G::kWaves * 4 * D * (int)sizeof(T);  // LDS bytes of the parts of one increment
-    static constexpr int kBwdTile = kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32
-                                    : kRowBytes * 16 <= 131072 ? 16 : kRowBytes * 8 <= 131072 ? 8 : 4;
+    static constexpr int kDP = D <= 4 ? 4 : D <= 8 ? 8 : 16;  // letters padded to whole 16-byte pieces
+    static constexpr bool kSlab = sizeof(T) == 4 && D <= 15 && !G::kSplit && G::kWaves <= 4;
+    static constexpr int kGroups = kDP / 4;        // 16-byte pieces per lane and increment
+    static constexpr int kSubTile = 32 / kDP;      // increments that wait in the slab: 8, 4 or 2 (8 KB per wave)
+    static constexpr int kSlabElems = kSlab ? G::kWaves * kSubTile * kWave * kDP : 4;
+    static constexpr int kParts = kSlab ? 8 : 4;
+    static constexpr int kLetters = kSlab ? kDP : D;  // cells of one increment in a row of `sg`
+    // LDS bytes of the parts of one increment
+    static constexpr int kRowBytes = G::kWaves * kParts * kLetters * (int)sizeof(T);
+    static constexpr int kBwdTile =
+        kSlab ? (kRowBytes * 32 <= 8192 ? 32 : kRowBytes * 16 <= 8192 ? 16 : 8)
+              : (kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32
+                 : kRowBytes * 16 <= 131072 ? 16 : kRowBytes * 8 <= 131072 ? 8 : 4);
     static constexpr int kStage = kBwdTile * KS * D;
     static constexpr int kSums = G::kWaves * kParts;
-    static constexpr int kSumRow = kBwdTile * D;
+    static constexpr int kSumRow = kBwdTile * kLetters;
     // fp64: the chain's P terms reach their letters through LDS (a row of D cells per lane, letter-major so that
     // a wave's accesses never share a bank).  A lane's prefix never changes, so it only ever touches the same
     // P cells and the others stay zero: P LDS adds, D loads and P clearing stores replace 3 * P * D selects and
@@ -1148,7 +1171,7 @@ __device__ __forceinline__ void dense_backward_body(
     const int tid,      // index of the thread within its block
     T (&sdx)[BackwardShape<T, D, N, P>::kStage],
     T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
-    T (&cells)[BackwardShape<T, D, N, P>::kCells]) {
+    T (&cells)[BackwardShape<T, D, N, P>::kCells], T (&slab)[BackwardShape<T, D, N, P>::kSlabElems], T (&carry)[D]) {
     using G = Geometry<D, N, P, sizeof(T)>;
     using BS = BackwardShape<T, D, N, P>;
     constexpr int KS = N - P;
@@ -1174,7 +1197,18 @@ __device__ __forceinline__ void dense_backward_body(
         for (int k = 0; k < D; ++k) my_cells[k * G::kBlock] = T(0);
     }
 
-    const int64_t unit = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
+    int64_t unit = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
+    if constexpr (CHUNKED && G::kUnitBlocks == 1) {
+        // Consecutive blocks go to the eight XCDs in turn, each with an L2 of its own.  The chunks of a row read the
+        // same upstream gradient, so they are dealt to one XCD: block b = 8 q + x works on the q-th unit of the
+        // rows x, x + 8, x + 16, ... (as long as whole groups of eight rows remain).
+        const int64_t total = (int64_t)gridDim.x, per_group = 8 * (int64_t)chunks;
+        if (unit < total / per_group * per_group) {
+            const int64_t group = unit / per_group, in_group = unit - group * per_group;
+            const int64_t x = in_group % 8, q = in_group / 8;
+            unit = (group * 8 + x) * chunks + q;
+        }
+    }
     const int64_t row = unit / chunks;
     const int c = (int)(unit - row * chunks);
     const int64_t b = row / shape.W, w = row - b * shape.W;
@@ -1196,7 +1230,16 @@ __device__ __forceinline__ void dense_backward_body(
         // adjoint at the right edge of the chunk: the upstream gradient contracted with the signature of
         // everything to the right of the chunk
         const SubWords<D, P> sw(u);
-        contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
+        // The lanes read the row of suffix products at addresses of their own, each entry several times over
+        // the block: where the slab has room for it the row goes there first, in one coalesced copy.
+        constexpr bool kStageEdge = BS::kSlab && RowStager<T, (int)G::kLowSize, G::kBlock>::kPadded <= BS::kSlabElems;
+        if constexpr (kStageEdge) {
+            copy_row<T, (int)G::kLowSize, G::kBlock>(edgeZ + unit * G::kLowSize, &slab[0], tid);
+            lds_barrier();
+            contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, &slab[0], sw);
+        } else {
+            contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
+        }
     } else {
         load_state<T, D, P, N - 1, kAS, KF>(sig + row * G::kSigSize, pu, active, a, asub, a0);
     }
@@ -1240,9 +1283,15 @@ __device__ __forceinline__ void dense_backward_body(
 
     const int64_t len = end - begin;
     const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
-    for (int64_t ti = ntiles - 1; ti >= 0; --ti) {
-        const int64_t t0 = begin + ti * kBwdTile;
-        const int nt = (int)((end - t0) < kBwdTile ? (end - t0) : kBwdTile);
+    // A chunk that writes the path gradient itself (kToPath) owns the points begin .. end - 1 of its row (the last
+    // chunk also the final point): dL/dx[t] = g[t-1] - g[t] with g the per-increment sums.  The sum of the last
+    // increment before the chunk, g[begin - 1], belongs to the chunk on the left; this chunk computes it again with
+    // one more step of its sweep (tile -1, the ghost step: the state after increment `begin` is exactly what that
+    // step needs), so every point has one writer, nothing is added in memory and the order of the sums is fixed.
+    const bool ghost = kToPath && len > 0 && begin > 0;
+    for (int64_t ti = ntiles - 1; ti >= (ghost ? -1 : 0); --ti) {
+        const int64_t t0 = ti < 0 ? begin - 1 : begin + ti * kBwdTile;
+        const int nt = ti < 0 ? 1 : (int)((end - t0) < kBwdTile ? (end - t0) : kBwdTile);
         const T *xw = x + t0 * D;
         lds_barrier();
         stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, tid);
@@ -1298,7 +1347,39 @@ __device__ __forceinline__ void dense_backward_body(
 #pragma unroll
                 for (int j = 0; j < P; ++j) my_cells[u[j] * G::kBlock] = T(0);
             }
-            if constexpr (kParts == 4) {
+            if constexpr (BS::kSlab) {
+                // the lane's terms of this increment go to its row of the wave's slab; the increment that completes
+                // a group of kSubTile sums the group over the lanes
+                using V4 = typename VecOf<T, 4>::type;
+                constexpr int kSub = BS::kSubTile, kGroups = BS::kGroups;
+                V4 *mine = reinterpret_cast<V4 *>(slab) +
+                           (size_t)(((wave * kSub + (tt & (kSub - 1))) * kWave + lane) * kGroups);
+#pragma unroll
+                for (int g = 0; g < kGroups; ++g) {
+                    V4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = 4 * g + e < D ? tot[4 * g + e < D ? 4 * g + e : 0] : T(0);
+                    mine[g] = v;
+                }
+                if ((tt & (kSub - 1)) == 0) {
+                    // (the LDS operations of a wave complete in order; the fence keeps the compiler from moving
+                    // the reads of other lanes' rows above the stores)
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    // lane -> (increment of the group, one eighth of the lanes, 16-byte piece of the letters)
+                    constexpr int kPer = kWave / kSub;  // lanes that share an increment: 8 * kGroups
+                    const int ttl = lane / kPer, part = (lane % kPer) / kGroups, piece = lane % kGroups;
+                    const V4 *rows = reinterpret_cast<const V4 *>(slab) +
+                                     (size_t)((wave * kSub + ttl) * kWave) * kGroups + piece;
+                    // source lanes 8 s + (part + s) % 8: the eight lanes that read together hit different banks
+                    V4 acc = rows[(size_t)(part & 7) * kGroups];
+#pragma unroll
+                    for (int s8 = 1; s8 < 8; ++s8) acc += rows[(size_t)(8 * s8 + ((part + s8) & 7)) * kGroups];
+                    if (tt + ttl < nt)  // (rows beyond the last increment of the tile hold nothing of this tile)
+                        reinterpret_cast<V4 *>(&sg[wave * 8 + part][0])[(tt + ttl) * kGroups + piece] = acc;
+                }
+            } else if constexpr (kParts == 4) {
                 // up to sixteen letters in one pass of exchanges (padded to a power of two with zeros), wider
                 // alphabets sixteen letters at a time; one store per row of 16 lanes and pass
                 constexpr int DP = D <= 2 ? 2 : D <= 4 ? 4 : D <= 8 ? 8 : 16;
@@ -1391,30 +1472,50 @@ __device__ __forceinline__ void dense_backward_body(
             }
         }
         lds_barrier();
+        // cell of (increment, letter) number idx in a row of `sg`
+        auto cell = [](int idx) { return BS::kLetters == D ? idx : (idx / D) * BS::kLetters + idx % D; };
         if constexpr (kToPath) {
             // Time-chunked, no windows: the path gradient dL/dx[t] = g[t-1] - g[t] leaves the kernel directly.
-            // Differences inside the tile are stored; the two ends of the tile are added to cells that the
-            // chunk-signature launch has cleared and that receive exactly one more term from the
-            // neighbouring tile (or none at the ends of the path), so the result does not depend on the order.
+            // Tiles are flushed from the right end of the chunk to its left end; `carry` holds g of the first
+            // increment of the tile flushed before (the one to the right), whose point is written now.
             for (int idx = tid; idx < nt * D; idx += G::kBlock) {
-                T v = sg[0][idx];
+                const int at = cell(idx);
+                T v = sg[0][at];
 #pragma unroll
-                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
-                sg[0][idx] = v;
+                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][at];
+                sg[0][at] = v;
             }
             lds_barrier();
             T *gp = grad_path + (b * shape.L + span.start + t0) * D;
-            for (int idx = tid; idx < nt * D; idx += G::kBlock) {
-                const T cur = sg[0][idx];
-                if (idx >= D) gp[idx] = sg[0][idx - D] - cur;
-                else atomicAdd(&gp[idx], -cur);
-                if (idx >= (nt - 1) * D) atomicAdd(&gp[idx + D], cur);
+            const bool rightmost = ti == ntiles - 1;
+            if (ti < 0) {
+                // ghost step: g[begin - 1] completes the first point of the chunk
+                for (int k = tid; k < D; k += G::kBlock) gp[D + k] = sg[0][cell(k)] - carry[k];
+            } else {
+                for (int idx = tid; idx < nt * D; idx += G::kBlock) {
+                    const T cur = sg[0][cell(idx)];
+                    if (idx >= D) gp[idx] = sg[0][cell(idx - D)] - cur;
+                    if (idx >= (nt - 1) * D) {
+                        // the point to the right of the tile: the final point of the row, or the first point of
+                        // the tile flushed before
+                        const int k = idx - (nt - 1) * D;
+                        if (!rightmost) gp[idx + D] = cur - carry[k];
+                        else if (c == chunks - 1) gp[idx + D] = cur;
+                    }
+                }
+                lds_barrier();
+                for (int k = tid; k < D; k += G::kBlock) {
+                    const T first = sg[0][cell(k)];
+                    if (ti == 0 && !ghost) gp[k] = -first;  // the first point of the row: nothing on its left
+                    carry[k] = first;
+                }
             }
         } else {
             for (int idx = tid; idx < nt * D; idx += G::kBlock) {
-                T v = sg[0][idx];
+                const int at = cell(idx);
+                T v = sg[0][at];
 #pragma unroll
-                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][idx];
+                for (int q = 1; q < G::kWaves * kParts; ++q) v += sg[q][at];
                 if constexpr (ACCUMULATE) {
                     atomicAdd(&ginc[t0 * D + idx], v);
                 } else {
@@ -1437,8 +1538,10 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     using BS = BackwardShape<T, D, N, P>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx[BS::kStage];
-    __shared__ T sg[BS::kSums][BS::kSumRow];
+    __shared__ __align__(16) T sg[BS::kSums][BS::kSumRow];
     __shared__ T cells[BS::kCells];
+    __shared__ __align__(16) T slab[BS::kSlabElems];
+    __shared__ T carry[D];  // kToPath: per-letter sums of the first increment of the tile flushed before
     using G = Geometry<D, N, P, sizeof(T)>;
     static_assert((G::kUnitBlocks == 1 || ACCUMULATE) && (!G::kOnePiece || (!CHUNKED && !BOUNDED)),
                   "a unit of several blocks is swept in one piece and adds its per-increment sums in memory");
@@ -1448,12 +1551,12 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value>(
-                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells);
+                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry);
         });
     } else {
         const int pu = G::kUnitBlocks > 1 ? tid + (int)(blockIdx.x % G::kUnitBlocks) * G::kBlock : tid;
         dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0>(path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape,
-                                                                chunks, grad_path, pu, tid, sdx, sg, cells);
+                                                                chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry);
     }
 }
 
@@ -1646,7 +1749,48 @@ constexpr bool group_fits() {
     return Geometry<D, N, P, sizeof(T)>::kBlock * GW <= 1024 && forward_lds_bytes<D, N, P, GW, T>() <= 64 * 1024;
 }
 
-template <typename T, int D, int N, int P, int PC>
+// A kernel that asks for more than 48 KB of dynamic LDS needs its limit raised first: once per kernel and device.
+template <typename K>
+hipError_t allow_dynamic_lds(K kernel, size_t bytes) {
+    static std::atomic<size_t> allowed[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && allowed[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes);
+    if (e == hipSuccess && tracked) allowed[dev].store(bytes, std::memory_order_release);
+    return e;
+}
+
+// Prefix products edgeA and suffix products edgeZ of the chunk signatures below the top level (dense_scan_kernel).
+template <typename T, int D, int N, int PS>
+hipError_t launch_scan(const T *chunk_low, T *edgeA, T *edgeZ, int64_t rows, int chunks, hipStream_t stream) {
+    using GC = Geometry<D, N, PS>;
+    // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
+    const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
+    const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
+    if (resident_bytes + fixed_bytes <= 150 * 1024) {
+        auto kernel = dense_scan_kernel<T, D, N, PS, true>;
+        if (resident_bytes > 48 * 1024) {
+            hipError_t e = allow_dynamic_lds(kernel, resident_bytes);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), resident_bytes, stream,
+                           chunk_low, edgeA, edgeZ, chunks, (T *)nullptr, (int64_t)0);
+    } else {
+        hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS, false>), dim3((unsigned)rows, 2),
+                           dim3(GC::kBlock + kCopyThreads), 0, stream, chunk_low, edgeA, edgeZ, chunks, (T *)nullptr,
+                           (int64_t)0);
+    }
+    return hipGetLastError();
+}
+
+// keep (optional): receives the prefix and suffix products of the chunk signatures below the top level, which the
+// time-chunked backward of the same call starts its chunks from: [rows, chunks, low] twice, the second array
+// pad256 bytes after the start of the first.
+template <typename T, int D, int N, int P, int PC, int PS>
 hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, T *keep,
                        void *workspace, hipStream_t stream) {
     using G = Geometry<D, N, P, sizeof(T)>;
@@ -1673,12 +1817,15 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     // chunks are swept GW to a block when that divides the chunk count and fits the block and LDS limits;
     // a row that fits one block goes straight to the output, without the combine launch
     T *chunk_sig = (T *)workspace;
+    // the chunks' own signatures below the top level, from which the products for the backward are made
+    T *chunk_low = keep ? (T *)((unsigned char *)workspace + pad256((size_t)rows * chunks * G::kSigSize * sizeof(T)))
+                        : (T *)nullptr;
     int groups = chunks;
     if constexpr (kBoundsOk) {
         if (bounds) {
             // bounded sweeps exist one chunk to a block only
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)(rows * chunks)),
-                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds, keep);
+                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds, chunk_low);
             groups = -1;
         }
     }
@@ -1687,7 +1834,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
             groups = chunks / 4;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 4>), dim3((unsigned)(rows * groups)),
                                dim3(G::kBlock * 4), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks,
-                               (T *)nullptr, (const int *)nullptr, keep);
+                               (T *)nullptr, (const int *)nullptr, chunk_low);
         }
     }
     if constexpr (group_fits<T, D, N, P, 2>()) {
@@ -1695,14 +1842,24 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
             groups = chunks / 2;
             hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 2>), dim3((unsigned)(rows * groups)),
                                dim3(G::kBlock * 2), 0, stream, path, groups == 1 ? sig : chunk_sig, shape, chunks,
-                               (T *)nullptr, (const int *)nullptr, keep);
+                               (T *)nullptr, (const int *)nullptr, chunk_low);
         }
     }
     if (groups == chunks)
         hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1>), dim3((unsigned)(rows * chunks)), dim3(G::kBlock), 0,
-                           stream, path, chunk_sig, shape, chunks, (T *)nullptr, (const int *)nullptr, keep);
+                           stream, path, chunk_sig, shape, chunks, (T *)nullptr, (const int *)nullptr, chunk_low);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || groups == 1) return e;
+    if (e != hipSuccess) return e;
+    if (keep) {
+        if constexpr (scan_fits<T, D, N, PS>()) {
+            T *edgeZ = (T *)((unsigned char *)keep + pad256((size_t)rows * chunks * G::kLowSize * sizeof(T)));
+            e = launch_scan<T, D, N, PS>((const T *)chunk_low, keep, edgeZ, rows, chunks, stream);
+            if (e != hipSuccess) return e;
+        } else {
+            return hipErrorNotSupported;  // such shapes are never cut into time chunks (dense_choice)
+        }
+    }
+    if (groups == 1) return hipSuccess;
     if (groups < 0) groups = chunks;
     if constexpr (kStaged)
         hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, true>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
@@ -1754,76 +1911,57 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         return hipErrorNotSupported;
     } else {
         const int64_t units = rows * chunks;
-        unsigned char *ws = (unsigned char *)workspace;
-        T *chunk_low = (T *)ws;
-        ws += pad256((size_t)units * G::kLowSize * sizeof(T));
-        T *dumpA = (T *)ws;
-        ws += pad256((size_t)units * G::kLowSize * sizeof(T));
-        T *dumpH = (T *)ws;
+        const size_t edge_bytes = pad256((size_t)units * G::kLowSize * sizeof(T));
+        const T *dumpA, *dumpH;
         if (kept) {
-            // the forward of this call kept its chunk signatures; the scan launch below clears the path gradient
-            chunk_low = const_cast<T *>(kept);
+            // the forward of this call left the prefix and suffix products of its chunk signatures
+            dumpA = kept;
+            dumpH = (const T *)((const unsigned char *)kept + edge_bytes);
         } else {
+            unsigned char *ws = (unsigned char *)workspace;
+            T *chunk_low = (T *)ws;
+            T *edgeA = (T *)(ws + edge_bytes), *edgeZ = (T *)(ws + 2 * edge_bytes);
             // chunk signatures below the top level: the depth N-1 forward kernel on the same units
-            // (without windows the same launch clears the path gradient, which the reverse sweep then fills in)
             // (the forward kernel needs a prefix shorter than its depth; the layout it writes does not depend on it)
             if constexpr (N == 2) {
                 hipLaunchKernelGGL(chunk_level1_kernel<T>, dim3((unsigned)units), dim3(kWave), 0, stream, path, chunk_low,
-                                   shape, chunks, accumulate ? (T *)nullptr : grad_path);
+                                   shape, chunks, (T *)nullptr);
             } else {
                 constexpr int PK = P <= N - 2 ? P : N - 2;
                 hipLaunchKernelGGL((dense_forward_kernel<T, D, N - 1, PK, 1>), dim3((unsigned)units),
                                    dim3(Geometry<D, N - 1, PK, sizeof(T)>::kBlock), 0, stream, path, chunk_low, shape, chunks,
-                                   accumulate ? (T *)nullptr : grad_path);
+                                   (T *)nullptr);
             }
             e = hipGetLastError();
             if (e != hipSuccess) return e;
+            e = launch_scan<T, D, N, PS>((const T *)chunk_low, edgeA, edgeZ, rows, chunks, stream);
+            if (e != hipSuccess) return e;
+            dumpA = edgeA;
+            dumpH = edgeZ;
         }
-        // without windows rows are paths: with kept chunk signatures the scan clears the path gradient
-        T *clear = (kept && !accumulate) ? grad_path : (T *)nullptr;
-        const int64_t clear_elems = shape.L * shape.d;
-        // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
-        const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
-        const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
-        if (resident_bytes + fixed_bytes <= 150 * 1024) {
-            auto kernel = dense_scan_kernel<T, D, N, PS, true>;
-            if (resident_bytes > 48 * 1024) {
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)resident_bytes);
-                if (e != hipSuccess) return e;
-            }
-            hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 2), dim3(GC::kBlock + kCopyThreads), resident_bytes, stream,
-                               (const T *)chunk_low, dumpA, dumpH, chunks, clear, clear_elems);
-        } else {
-            hipLaunchKernelGGL((dense_scan_kernel<T, D, N, PS, false>), dim3((unsigned)rows, 2),
-                               dim3(GC::kBlock + kCopyThreads), 0, stream, (const T *)chunk_low, dumpA, dumpH, chunks,
-                               clear, clear_elems);
-        }
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
         profile_bracket(true, stream);
         bool launched = false;
         if constexpr (kBoundsOk) {
             if (bounds) {
                 if (accumulate)
                     hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true, true>), dim3((unsigned)units),
-                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA,
-                                       (const T *)dumpH, grad_inc, shape, chunks, (T *)nullptr, bounds);
+                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA,
+                                       dumpH, grad_inc, shape, chunks, (T *)nullptr, bounds);
                 else
                     hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true, true>), dim3((unsigned)units),
-                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA,
-                                       (const T *)dumpH, grad_inc, shape, chunks, grad_path, bounds);
+                                       dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA,
+                                       dumpH, grad_inc, shape, chunks, grad_path, bounds);
                 launched = true;
             }
         }
         if (!launched) {
             if (accumulate)
                 hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units),
-                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
+                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA, dumpH,
                                    grad_inc, shape, chunks, (T *)nullptr);
             else
                 hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
-                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, (const T *)dumpA, (const T *)dumpH,
+                                   dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA, dumpH,
                                    grad_inc, shape, chunks, grad_path);
         }
         if (!accumulate) *wrote_path = true;
@@ -1924,11 +2062,15 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
         dc.bwd_chunks = (dc.embed && !dc.resweep && chunks < 2) ? 2 : chunks;
         dc.forward_workspace = dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
         dc.backward_workspace = (dc.resweep ? 2 : 1) * dc.dense_bytes + (dc.bounded ? kBoundsBytes : 0);
-        if (dc.fwd_chunks > 1) dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem);
+        // forward: the chunk signatures, and those below the top level from which a keeping forward makes the
+        // products its backward starts from; backward: the latter and the two arrays of products
+        if (dc.fwd_chunks > 1)
+            dc.forward_workspace += pad256((size_t)rows * dc.fwd_chunks * v.sig_size * elem) +
+                                    pad256((size_t)rows * dc.fwd_chunks * v.low_size * elem);
         if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
-        // the forward can hand its chunk signatures to the backward when both cut the rows the same way
+        // the forward can hand those products to the backward when both cut the rows the same way
         if (dc.bwd_chunks > 1 && dc.fwd_chunks == dc.bwd_chunks)
-            dc.keep_bytes = (size_t)rows * dc.bwd_chunks * v.low_size * elem;
+            dc.keep_bytes = 2 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
         if (dc.resweep) dc.keep_bytes = (size_t)rows * v.sig_size * elem;
         return dc;
     }
@@ -1995,7 +2137,8 @@ static_assert(PSIG_GROUP < kDenseGroups, "group index out of range");
 #define PSIG_CASE_FWD(I, D, N, P, PC, PS)                                                                         \
     case I:                                                                                                       \
         if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                      \
-            return run_forward<T, D, N, P, PC>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace, stream); \
+            return run_forward<T, D, N, P, PC, PS>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace,    \
+                                                   stream);                                                       \
         break;
 #define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
     case I:                                                                                                        \
