@@ -414,9 +414,30 @@ __device__ __forceinline__ Span unit_span(const SigShape &shape, int64_t w) {
 }
 
 // chunk c of `chunks` equal parts of a span: steps [begin, end)
+// (64-bit divisions are some thirty scalar instructions each, in front of every unit's first load: spans of less
+// than 2^31 steps, that is all spans met in practice, take one 32-bit division and small ones for the remainder)
 __device__ __forceinline__ void chunk_range(int64_t steps, int chunks, int c, int64_t &begin, int64_t &end) {
-    begin = steps * c / chunks;
-    end = steps * (c + 1) / chunks;
+    if (steps < (int64_t(1) << 31) && chunks <= 32768) {
+        // floor(steps * c / chunks) = q * c + floor(r * c / chunks) with steps = q * chunks + r
+        const unsigned q = (unsigned)steps / (unsigned)chunks, r = (unsigned)steps - q * (unsigned)chunks;
+        begin = (int64_t)q * c + (r * (unsigned)c) / (unsigned)chunks;
+        end = (int64_t)q * (c + 1) + (r * (unsigned)(c + 1)) / (unsigned)chunks;
+    } else {
+        begin = steps * c / chunks;
+        end = steps * (c + 1) / chunks;
+    }
+}
+
+// quotient and remainder of a block or row index (always below 2^31: a grid dimension) by a small positive divisor
+__device__ __forceinline__ void divide_index(int64_t index, int64_t by, int64_t &quotient, int64_t &remainder) {
+    if (index < (int64_t(1) << 31) && by < (int64_t(1) << 31)) {
+        const unsigned q = (unsigned)index / (unsigned)by;
+        quotient = q;
+        remainder = (unsigned)index - q * (unsigned)by;
+    } else {
+        quotient = index / by;
+        remainder = index - quotient * by;
+    }
 }
 
 constexpr int kTile = 64;  // increments staged in LDS at a time
@@ -728,16 +749,18 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
 
     const int groups = chunks / GW;  // blocks per row
     const int64_t blk = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
-    const int64_t row = blk / groups;
-    const int c = (int)(blk - row * groups) * GW + part;
-    const int64_t b = row / shape.W, w = row - b * shape.W;
+    int64_t row, group_of_row, b, w;
+    divide_index(blk, groups, row, group_of_row);
+    const int c = (int)group_of_row * GW + part;
+    divide_index(row, shape.W, b, w);
     const Span span = unit_span(shape, w);
     int64_t begin, end;
     chunk_range(span.steps, chunks, c, begin, end);
     const T *x = path + (b * shape.L + span.start) * D;
     // every chunk of the row has floor or ceil of steps/chunks increments: the longest sets the number
     // of tile rounds for the whole block, so all threads meet at the same barriers
-    const int64_t longest = (span.steps + chunks - 1) / chunks;
+    int64_t longest, longest_rest;
+    divide_index(span.steps + chunks - 1, chunks, longest, longest_rest);
     if constexpr (GW == 1) {
         if (zero_rows) {
             const int64_t points = end - begin + (c == chunks - 1 ? 1 : 0);
@@ -877,60 +900,97 @@ struct RowStager {
 #pragma unroll
         for (int i = 0; i < kPer; ++i) v[i * BLOCK + (int)threadIdx.x] = regs[i];
     }
+    // the same into a buffer of exactly COUNT elements
+    __device__ __forceinline__ void commit_exact(T *dst) const {
+        V *v = reinterpret_cast<V *>(dst);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int idx = i * BLOCK + (int)threadIdx.x;
+            if (idx < kVecs) v[idx] = regs[i];
+        }
+    }
 };
 
 // product of the chunk signatures of one row, left to right.  Lanes sit on prefixes of length P (one
 // more letter than in the sweep kernels, for more lanes per row).  Chunks are fetched into registers
 // kAhead products before they are needed and handed over through a double buffer in LDS.
-template <typename T, int D, int N, int P, bool STAGED>
-__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
-    dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks) {
+// BLOCK: threads that work on a row together (all lanes of the row, or a part of them when the row is spread over
+// several blocks, each of which stages the whole right factor for itself)
+template <typename T, int D, int N, int P, int BLOCK = Geometry<D, N, P>::kBlock>
+struct CombineShape {
     using G = Geometry<D, N, P>;
-    constexpr int kStage = STAGED ? RowStager<T, (int)G::kSigSize, G::kBlock>::kPadded : 4;
+    static constexpr int kStage = RowStager<T, (int)G::kSigSize, BLOCK>::kPadded;
+    static constexpr size_t kBytes = 2 * (size_t)kStage * sizeof(T);
+};
+
+// (the first BLOCK threads of the block, on the lanes lane_base .. lane_base + BLOCK - 1 of the row; sB: two buffers
+// of CombineShape::kStage elements)
+template <typename T, int D, int N, int P, int BLOCK = Geometry<D, N, P>::kBlock>
+__device__ __forceinline__ void combine_staged(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks,
+                                               int64_t row, T *sB0, T *sB1, int lane_base = 0) {
+    using G = Geometry<D, N, P>;
     constexpr int kAhead = 3;
-    __shared__ __align__(16) T sB[2][kStage];
-    // without staging the lanes are independent: the row may then be spread over gridDim.y blocks
-    const int pu = STAGED ? (int)threadIdx.x : (int)(blockIdx.y * blockDim.x + threadIdx.x);
+    const int pu = lane_base + (int)threadIdx.x;
     const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
     int u[P];
     prefix_letters<D, P>(active ? pu : 0, u);
     const SubWords<D, P> sw(u);
-    const int64_t row = blockIdx.x;
     const T *rows = chunk_sig + row * chunks * G::kSigSize;
     T a[P + 1];
     T sub[G::kFwdSub];
     load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
-    if constexpr (STAGED) {
-        // Register set q holds chunk c with (c - 1) % kAhead == q.  Fetches past the last chunk re-read the
-        // last chunk instead of branching, so the waits on them stay exact counts.
-        const int last = chunks - 1;
-        RowStager<T, (int)G::kSigSize, G::kBlock> stager[kAhead];
+    // Register set q holds chunk c with (c - 1) % kAhead == q.  Fetches past the last chunk re-read the
+    // last chunk instead of branching, so the waits on them stay exact counts.
+    const int last = chunks - 1;
+    RowStager<T, (int)G::kSigSize, BLOCK> stager[kAhead];
+    static_for<0, kAhead>([&](auto qc) {
+        constexpr int q = decltype(qc)::value;
+        stager[q].fetch(rows + (int64_t)(1 + q < last ? 1 + q : last) * G::kSigSize);
+    });
+    stager[0].commit(sB1);
+    stager[0].fetch(rows + (int64_t)(1 + kAhead < last ? 1 + kAhead : last) * G::kSigSize);
+    lds_barrier();
+    for (int base = 1; base < chunks; base += kAhead) {
         static_for<0, kAhead>([&](auto qc) {
             constexpr int q = decltype(qc)::value;
-            stager[q].fetch(rows + (int64_t)(1 + q < last ? 1 + q : last) * G::kSigSize);
+            constexpr int qn = (q + 1) % kAhead;  // register set of the next chunk
+            const int c = base + q;
+            if (c < chunks) {
+                apply_right<T, D, P, N, G::kFwdSub>(a, sub, (c & 1) ? sB1 : sB0, sw);
+                stager[qn].commit(((c + 1) & 1) ? sB1 : sB0);
+                const int nxt = c + 1 + kAhead;
+                stager[qn].fetch(rows + (int64_t)(nxt < last ? nxt : last) * G::kSigSize);
+                lds_barrier();
+            }
         });
-        stager[0].commit(sB[1]);
-        stager[0].fetch(rows + (int64_t)(1 + kAhead < last ? 1 + kAhead : last) * G::kSigSize);
-        lds_barrier();
-        for (int base = 1; base < chunks; base += kAhead) {
-            static_for<0, kAhead>([&](auto qc) {
-                constexpr int q = decltype(qc)::value;
-                constexpr int qn = (q + 1) % kAhead;  // register set of the next chunk
-                const int c = base + q;
-                if (c < chunks) {
-                    apply_right<T, D, P, N, G::kFwdSub>(a, sub, sB[c & 1], sw);
-                    stager[qn].commit(sB[(c + 1) & 1]);
-                    const int nxt = c + 1 + kAhead;
-                    stager[qn].fetch(rows + (int64_t)(nxt < last ? nxt : last) * G::kSigSize);
-                    lds_barrier();
-                }
-            });
-        }
-    } else {
-        for (int c = 1; c < chunks; ++c)
-            apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
     }
     if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
+}
+
+template <typename T, int D, int N, int P, bool STAGED>
+__global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
+    dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks) {
+    using G = Geometry<D, N, P>;
+    constexpr int kStage = STAGED ? CombineShape<T, D, N, P>::kStage : 4;
+    __shared__ __align__(16) T sB[2][kStage];
+    if constexpr (STAGED) {
+        combine_staged<T, D, N, P>(chunk_sig, sig, chunks, (int64_t)blockIdx.x, sB[0], sB[1]);
+    } else {
+        // without staging the lanes are independent: the row is spread over gridDim.y blocks
+        const int pu = (int)(blockIdx.y * blockDim.x + threadIdx.x);
+        const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
+        int u[P];
+        prefix_letters<D, P>(active ? pu : 0, u);
+        const SubWords<D, P> sw(u);
+        const int64_t row = blockIdx.x;
+        const T *rows = chunk_sig + row * chunks * G::kSigSize;
+        T a[P + 1];
+        T sub[G::kFwdSub];
+        load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
+        for (int c = 1; c < chunks; ++c)
+            apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
+        if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1092,6 +1152,135 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock + kCopyThreads))
     }
 }
 
+// The scan and the product of the partial signatures of the forward sweep in one launch: three chains of dependent
+// products per row, in blocks that are small enough for two of them to share a CU, so that they run side by side
+// (as launches of their own, the 128 to 256 blocks of each leave most of the device idle, one after the other).
+//   blockIdx.y == 0:  edgeA_c = S_0 (x) .. (x) S_c
+//   blockIdx.y == 1:  edgeZ_c = S_{c+1} (x) .. (x) S_{C-1}
+//   blockIdx.y >= 2:  the signature of the row from its `groups` partial products (combine_staged), the lanes of
+//                     the row dealt to one or more blocks
+// The scans work like dense_scan_kernel with all rows in LDS, except that only `resident` chunk rows have a place
+// there: the up to kEdgeExtra rows that a scan uses last are fetched into registers at the start and take the
+// places of the rows used first once those have been read.  (A deeper pipeline of fetches through registers is not
+// an option: after the first branch the compiler waits for every outstanding load before it uses any.)
+constexpr int kEdgeExtra = 3;
+
+template <typename T, int D, int N, int PS, int PC>
+struct EdgesShape {
+    using GS = Geometry<D, N, PS>;
+    using GC = Geometry<D, N, PC>;
+    static constexpr int kLow = (int)GS::kLowSize;
+    static constexpr int kScanThreads = GS::kBlock + kCopyThreads;
+    // the combine's lanes in blocks of at most 512 threads (two such blocks share a CU whatever their registers)
+    static constexpr int kCombineBlock = GC::kBlock <= 512 ? GC::kBlock : 512;
+    static constexpr int kCombineParts = GC::kBlock / kCombineBlock;
+    static constexpr int kThreads = kCombineBlock > kScanThreads ? kCombineBlock : kScanThreads;
+    static constexpr size_t kRowBytes = (size_t)kLow * sizeof(T);
+    static constexpr size_t kStaticBytes = 2 * kRowBytes;  // the double buffer of the scans
+    static constexpr size_t kCombineBytes = CombineShape<T, D, N, PC, kCombineBlock>::kBytes;  // staging of the combine
+    static constexpr size_t kBudget = 78 * 1024;           // two blocks to a CU
+    static constexpr bool kUsable = kThreads <= 512 && GC::kBlock % kCombineBlock == 0 && N >= 2 && !GS::kOnePiece &&
+                                    kRowBytes % 16 == 0 && kStaticBytes + kCombineBytes <= kBudget;
+};
+
+template <typename T, int D, int N, int P, bool ascending>
+__device__ __forceinline__ void scan_resident(const T *__restrict__ chunk_low, T *__restrict__ edges, int chunks,
+                                              int resident, int64_t row, T *sAll, T *sOut0, T *sOut1) {
+    using G = Geometry<D, N, P>;
+    using Stager = RowStager<T, (int)G::kLowSize, G::kBlock>;
+    constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
+    constexpr int kLow = (int)G::kLowSize;
+    constexpr int kThreads = G::kBlock + kCopyThreads;
+    const bool copier = (int)threadIdx.x >= G::kBlock;
+    const int ctid = (int)threadIdx.x - G::kBlock;
+    const int pu = copier ? 0 : (int)threadIdx.x;
+    const bool active = !copier && ((G::kLanes == G::kBlock) || pu < G::kLanes);
+    int u[P];
+    prefix_letters<D, P>(active ? pu : 0, u);
+    const SubWords<D, P> sw(u);
+    const T *rows = chunk_low + row * chunks * kLow;
+    T *edge = edges + row * chunks * kLow;
+    const int last = chunks - 1;
+    // rows in the order of their use: edgeA multiplies the chunks 1, 2, .. onto chunk 0, edgeZ takes the chunks
+    // last, last - 1, .., 1 as the left factor of its running product
+    const int used = last;
+    auto chunk_of = [&](int j) { return ascending ? 1 + j : last - j; };
+    const int held = resident < used ? resident : used;
+    Stager extra[kEdgeExtra];
+    if (!copier) {
+        static_for<0, kEdgeExtra>([&](auto ec) {
+            constexpr int e = decltype(ec)::value;
+            const int j = held + e < used ? held + e : used - 1;
+            extra[e].fetch(rows + (int64_t)chunk_of(j) * kLow);
+        });
+    }
+    // (unrolled so that the loads of several rows are in flight together: one memory latency for the burst)
+#pragma unroll 8
+    for (int j = 0; j < held; ++j)
+        copy_row<T, kLow, kThreads>(rows + (int64_t)chunk_of(j) * kLow, sAll + (int64_t)j * kLow, (int)threadIdx.x);
+    T a[P + 1];
+    T asub[kAS];
+    if (!copier) {
+        if (ascending) {
+            load_state<T, D, P, N - 1, kAS>(rows, pu, active, a, asub);
+            if (active) store_state<T, D, P, N - 1, kAS>(sOut0, pu, a, asub);
+        } else {
+            // the product to the right of the last chunk is the identity (all coefficients zero)
+            for (int idx = threadIdx.x; idx < kLow; idx += G::kBlock) ((last & 1) ? sOut1 : sOut0)[idx] = T(0);
+        }
+    }
+    lds_barrier();
+    for (int j = 0; j < used; ++j) {
+        const int c = chunk_of(j);
+        const T *slot = sAll + (int64_t)(j < held ? j : j - held) * kLow;
+        if (!copier) {
+            // the row of the round before has been read by everyone: its place takes the row that comes `held` later
+            static_for<0, kEdgeExtra>([&](auto ec) {
+                constexpr int e = decltype(ec)::value;
+                if (j == e + 1 && held + e < used) extra[e].commit_exact(sAll + (int64_t)e * kLow);
+            });
+            if (ascending) {
+                apply_right<T, D, P, N - 1, kAS>(a, asub, slot, sw);
+                if (active) store_state<T, D, P, N - 1, kAS>((c & 1) ? sOut1 : sOut0, pu, a, asub);
+            } else {
+                // Z_{c-1} = S_c (x) Z_c
+                load_state<T, D, P, N - 1, kAS>(slot, pu, active, a, asub);
+                apply_right<T, D, P, N - 1, kAS>(a, asub, (c & 1) ? sOut1 : sOut0, sw);
+                if (active) store_state<T, D, P, N - 1, kAS>(((c - 1) & 1) ? sOut1 : sOut0, pu, a, asub);
+            }
+        } else {
+            if (ascending) copy_row_out<T, kLow>(((c - 1) & 1) ? sOut1 : sOut0, edge + (int64_t)(c - 1) * kLow, ctid);
+            else copy_row_out<T, kLow>((c & 1) ? sOut1 : sOut0, edge + (int64_t)c * kLow, ctid);
+        }
+        lds_barrier();
+    }
+    if (copier) {
+        if (ascending) copy_row_out<T, kLow>((last & 1) ? sOut1 : sOut0, edge + (int64_t)last * kLow, ctid);
+        else copy_row_out<T, kLow>(sOut0, edge, ctid);
+    }
+}
+
+template <typename T, int D, int N, int PS, int PC>
+__global__ void __launch_bounds__((EdgesShape<T, D, N, PS, PC>::kThreads))
+    dense_edges_kernel(const T *__restrict__ chunk_low, T *__restrict__ edgeA, T *__restrict__ edgeZ, int chunks,
+                       int resident, const T *__restrict__ partial, T *__restrict__ sig, int groups) {
+    using ES = EdgesShape<T, D, N, PS, PC>;
+    extern __shared__ __align__(16) unsigned char edges_smem[];
+    __shared__ __align__(16) T sOut[2][ES::kLow];
+    T *dyn = reinterpret_cast<T *>(edges_smem);
+    const int64_t row = blockIdx.x;
+    if (blockIdx.y >= 2) {
+        if ((int)threadIdx.x >= ES::kCombineBlock) return;
+        combine_staged<T, D, N, PC, ES::kCombineBlock>(partial, sig, groups, row, dyn,
+                                                       dyn + CombineShape<T, D, N, PC, ES::kCombineBlock>::kStage,
+                                                       ((int)blockIdx.y - 2) * ES::kCombineBlock);
+        return;
+    }
+    if ((int)threadIdx.x >= ES::kScanThreads) return;
+    if (blockIdx.y == 0) scan_resident<T, D, N, PS, true>(chunk_low, edgeA, chunks, resident, row, dyn, sOut[0], sOut[1]);
+    else scan_resident<T, D, N, PS, false>(chunk_low, edgeZ, chunks, resident, row, dyn, sOut[0], sOut[1]);
+}
+
 // Depth 2: the signature of a chunk below the top level is its level 1, the sum of its increments.  One block
 // per (row, chunk); zero_rows as in dense_forward_kernel (the block also clears the points of its chunk in a
 // [B, L, d] buffer, the last chunk of a row the final point too).
@@ -1099,9 +1288,10 @@ template <typename T>
 __global__ void __launch_bounds__(kWave) chunk_level1_kernel(const T *__restrict__ path, T *__restrict__ chunk_low,
                                                              SigShape shape, int chunks, T *__restrict__ zero_rows) {
     const int64_t unit = blockIdx.x;
-    const int64_t row = unit / chunks;
-    const int c = (int)(unit - row * chunks);
-    const int64_t b = row / shape.W, w = row - b * shape.W;
+    int64_t row, chunk_of_row, b, w;
+    divide_index(unit, chunks, row, chunk_of_row);
+    const int c = (int)chunk_of_row;
+    divide_index(row, shape.W, b, w);
     const Span span = unit_span(shape, w);
     int64_t begin, end;
     chunk_range(span.steps, chunks, c, begin, end);
@@ -1202,16 +1392,18 @@ __device__ __forceinline__ void dense_backward_body(
         // Consecutive blocks go to the eight XCDs in turn, each with an L2 of its own.  The chunks of a row read the
         // same upstream gradient, so they are dealt to one XCD: block b = 8 q + x works on the q-th unit of the
         // rows x, x + 8, x + 16, ... (as long as whole groups of eight rows remain).
-        const int64_t total = (int64_t)gridDim.x, per_group = 8 * (int64_t)chunks;
-        if (unit < total / per_group * per_group) {
-            const int64_t group = unit / per_group, in_group = unit - group * per_group;
-            const int64_t x = in_group % 8, q = in_group / 8;
-            unit = (group * 8 + x) * chunks + q;
+        // (grid dimensions are below 2^31: 32-bit arithmetic)
+        const unsigned total = gridDim.x, per_group = 8u * (unsigned)chunks, at = (unsigned)unit;
+        if (at < total / per_group * per_group) {
+            const unsigned group = at / per_group, in_group = at - group * per_group;
+            const unsigned x = in_group & 7u, q = in_group >> 3;
+            unit = ((int64_t)group * 8 + x) * chunks + q;
         }
     }
-    const int64_t row = unit / chunks;
-    const int c = (int)(unit - row * chunks);
-    const int64_t b = row / shape.W, w = row - b * shape.W;
+    int64_t row, chunk_of_row, b, w;
+    divide_index(unit, chunks, row, chunk_of_row);
+    const int c = (int)chunk_of_row;
+    divide_index(row, shape.W, b, w);
     const Span span = unit_span(shape, w);
     int64_t begin, end;
     chunk_range(span.steps, chunks, c, begin, end);
@@ -1768,6 +1960,7 @@ hipError_t allow_dynamic_lds(K kernel, size_t bytes) {
 template <typename T, int D, int N, int PS>
 hipError_t launch_scan(const T *chunk_low, T *edgeA, T *edgeZ, int64_t rows, int chunks, hipStream_t stream) {
     using GC = Geometry<D, N, PS>;
+
     // all chunk rows of a row go to LDS at once when they fit (a little under the 160 KB of a CU)
     const size_t resident_bytes = (size_t)chunks * GC::kLowSize * sizeof(T);
     const size_t fixed_bytes = 2 * GC::kLowSize * sizeof(T) + 1024;
@@ -1850,9 +2043,30 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            stream, path, chunk_sig, shape, chunks, (T *)nullptr, (const int *)nullptr, chunk_low);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if (groups < 0) groups = chunks;
     if (keep) {
         if constexpr (scan_fits<T, D, N, PS>()) {
             T *edgeZ = (T *)((unsigned char *)keep + pad256((size_t)rows * chunks * G::kLowSize * sizeof(T)));
+            if constexpr (kStaged && EdgesShape<T, D, N, PS, PC>::kUsable) {
+                // the products for the backward and the product of the partial signatures in one launch, when
+                // all but kEdgeExtra of the chunk rows of a scan fit the LDS share of a block
+                using ES = EdgesShape<T, D, N, PS, PC>;
+                const size_t room = ES::kBudget - ES::kStaticBytes;
+                const int used = chunks - 1;
+                const int resident = (int)std::min<size_t>((size_t)used, room / ES::kRowBytes);
+                if (groups > 1 && resident >= 2 && used - resident <= kEdgeExtra) {
+                    const size_t dynamic = std::max((size_t)resident * ES::kRowBytes, ES::kCombineBytes);
+                    auto kernel = dense_edges_kernel<T, D, N, PS, PC>;
+                    if (dynamic > 48 * 1024) {
+                        e = allow_dynamic_lds(kernel, dynamic);
+                        if (e != hipSuccess) return e;
+                    }
+                    hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 2 + ES::kCombineParts), dim3(ES::kThreads),
+                                       dynamic, stream, (const T *)chunk_low, keep, edgeZ, chunks, resident,
+                                       (const T *)chunk_sig, sig, groups);
+                    return hipGetLastError();
+                }
+            }
             e = launch_scan<T, D, N, PS>((const T *)chunk_low, keep, edgeZ, rows, chunks, stream);
             if (e != hipSuccess) return e;
         } else {
@@ -1860,7 +2074,6 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
         }
     }
     if (groups == 1) return hipSuccess;
-    if (groups < 0) groups = chunks;
     if constexpr (kStaged)
         hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, true>), dim3((unsigned)rows), dim3(GC::kBlock), 0, stream,
                            (const T *)chunk_sig, sig, groups);
