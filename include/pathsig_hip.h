@@ -176,6 +176,11 @@ int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const vo
  *                     1/8 of the dense one, or the dense sweep is estimated cheaper), 0 = none, n > 0 = those whose
  *                     top level keeps at least 1/n of the dense one (PATHSIG_EMBED_SHARE)
  *   "tiled"           0 = every call takes the per-word kernels, whatever its shape (PATHSIG_NO_TILED sets 0)
+ *   "deep_fp64"       1 (default) = a PATHSIG_F32 backward of depth 9 or more runs in fp64 on copies of the path
+ *                     and of grad_sig (its workspace holds them), sweeps the signature again in fp64 and rounds the
+ *                     path gradient at the end, unless it is a dense call of depth 9 cut into four time chunks or
+ *                     more; 0 = in fp32 like any other call, two to three times as fast and off by up to 3.5e-5 of
+ *                     the largest gradient at depth 12 (PATHSIG_NO_DEEP_FP64 sets 0)
  * Returns PATHSIG_ERR_ARGUMENT for an unknown name or a value out of range.
  */
 int pathsig_set_option(const char *name, int64_t value);

@@ -37,14 +37,15 @@ int64_t env_int(const char *name, int64_t fallback) {
 
 // Plain integers behind relaxed atomics: a setter on one thread and a call on another see whole values.
 struct OptionCells {
-    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share, tiled;
+    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share, tiled, deep_fp64;
     OptionCells()
         : chunks(env_int("PATHSIG_CHUNKS", 0)),
           letter_bounds(getenv("PATHSIG_NO_LETTER_BOUNDS") ? 0 : 1),
           logsig_scatter(env_int("PATHSIG_LOGSIG_SCATTER", 0) == 1 ? 1 : 0),
           batch_tile(env_int("PATHSIG_BATCH_TILE", 0)),
           embed_share(env_int("PATHSIG_EMBED_SHARE", -1)),
-          tiled(getenv("PATHSIG_NO_TILED") ? 0 : 1) {}
+          tiled(getenv("PATHSIG_NO_TILED") ? 0 : 1),
+          deep_fp64(getenv("PATHSIG_NO_DEEP_FP64") ? 0 : 1) {}
 };
 OptionCells &option_cells() {
     static OptionCells cells;  // the environment is read here, once
@@ -61,6 +62,7 @@ const Options &options() {
     snapshot.batch_tile = c.batch_tile.load(std::memory_order_relaxed);
     snapshot.embed_share = c.embed_share.load(std::memory_order_relaxed);
     snapshot.tiled = c.tiled.load(std::memory_order_relaxed);
+    snapshot.deep_fp64 = c.deep_fp64.load(std::memory_order_relaxed);
     return snapshot;
 }
 
@@ -330,6 +332,39 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     return PATHSIG_OK;
 }
 
+// Deep fp32 calls.  The reverse sweep rebuilds the signature of every earlier time by multiplying with exp(-dx_t),
+// and the gradient of a top-level coefficient sums thousands of terms of mixed sign: from depth 9 on, fp32 rounding
+// in those two places passes 1e-5 of the largest gradient (over a span of increments of size one, swept in one
+// piece: 1.0e-5 to 1.5e-5 at depth 9, up to 3.5e-5 at depth 12).  Such a backward runs in fp64 on copies of the
+// path and of the upstream gradient, sweeps the signature again in fp64 (rolled back over such a span, the rounding
+// of the fp32 signature alone shows as 1.4e-5 in the gradient at depth 10) and rounds the path gradient at the end;
+// the forward call stays in fp32.  Exempt: dense calls of depth 9 that are cut into four time chunks or more, which
+// stay below 1e-5 in fp32.
+__global__ void __launch_bounds__(256) widen_kernel(const float *__restrict__ src, double *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+__global__ void __launch_bounds__(256) narrow_kernel(const double *__restrict__ src, float *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        dst[i] = (float)src[i];
+}
+unsigned convert_blocks(int64_t n) { return (unsigned)std::min<int64_t>((n + 255) / 256, 16384); }
+
+bool backward_in_fp64(int dtype, int depth, const DenseChoice &dc) {
+    if (dtype != PATHSIG_F32 || depth < 9 || options().deep_fp64 == 0) return false;
+    return depth >= 10 || !(dc.usable && !dc.embed && dc.bwd_chunks >= 4);
+}
+
+struct DeepLayout {
+    size_t path_bytes, sig_bytes, total;  // two buffers of each size, then the workspace of the fp64 call
+};
+DeepLayout deep_layout(int64_t B, int64_t L, int64_t d, int64_t rows, int64_t sig_size, size_t inner) {
+    DeepLayout lay;
+    lay.path_bytes = align_up((size_t)(B * L * d) * sizeof(double));
+    lay.sig_bytes = align_up((size_t)(rows * sig_size) * sizeof(double));
+    lay.total = 2 * lay.path_bytes + 2 * lay.sig_bytes + inner;
+    return lay;
+}
+
 int check_logsig(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
     if (dtype != PATHSIG_F32 && dtype != PATHSIG_F64) {
         set_error("dtype must be PATHSIG_F32 or PATHSIG_F64 (got %d)", dtype);
@@ -394,7 +429,8 @@ int pathsig_set_option(const char *name, int64_t value) {
         option_cells().embed_share.store(value, std::memory_order_relaxed);
     } else if (!strcmp(name, "tiled") && (value == 0 || value == 1)) {
         option_cells().tiled.store(value, std::memory_order_relaxed);
-
+    } else if (!strcmp(name, "deep_fp64") && (value == 0 || value == 1)) {
+        option_cells().deep_fp64.store(value, std::memory_order_relaxed);
     } else {
         set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
         return PATHSIG_ERR_ARGUMENT;
@@ -461,6 +497,11 @@ size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d
     if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
     const DenseChoice dc =
         dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
+    if (backward_in_fp64(dtype, depth, dc)) {
+        const size_t inner = std::max(pathsig_sig_backward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, W),
+                                      pathsig_sig_forward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, W));
+        return deep_layout(B, L, d, B * (W > 0 ? W : 1), plan.sig_size, inner).total;
+    }
     const bool words_kernel = !dc.usable && !batch_backward_usable(elem_size(dtype), B, d, W > 0 ? W : 1);
     const bool batch_wide = !dc.usable && !words_kernel && batch_wide_sums(elem_size(dtype), plan);
     return inc_buffer_bytes(elem_size(dtype), B, L, d, words_kernel || batch_wide) +
@@ -543,6 +584,56 @@ int pathsig_sig_backward_kept(const void *path, const void *sig, const void *gra
         if (!empty) {
             set_error("sig and grad_sig must not be NULL");
             return PATHSIG_ERR_ARGUMENT;
+        }
+    }
+    if (dtype == PATHSIG_F32 && depth >= 9 && B > 0) {
+        LevelPlan plan;
+        bool all_dense;
+        rc = build_plan(d, depth, level_sizes, n_encoded, encoded_words != nullptr, &plan, &all_dense);
+        if (rc != PATHSIG_OK) return rc;
+        const int64_t rows = B * (windows ? W : 1);
+        const DenseChoice dc =
+            dense_choice(sizeof(float), d, depth, all_dense, level_sizes, B, L, windows ? W : 1, windows != nullptr);
+        if (backward_in_fp64(dtype, depth, dc)) {
+            // (the fp32 signature of the call, rounded, is no state to roll back from: the signature is swept again
+            // in fp64; what a keeping forward left is in fp32 and stays unused)
+            const size_t inner =
+                std::max(pathsig_sig_backward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, windows ? W : 0),
+                         pathsig_sig_forward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, windows ? W : 0));
+            const DeepLayout lay = deep_layout(B, L, d, rows, plan.sig_size, inner);
+            if (!workspace || workspace_bytes < lay.total) {
+                set_error("workspace too small: need %zu bytes, got %zu", lay.total, workspace_bytes);
+                return PATHSIG_ERR_WORKSPACE;
+            }
+            hipStream_t st = (hipStream_t)stream;
+            unsigned char *at = (unsigned char *)workspace;
+            double *path64 = (double *)at, *gpath64 = (double *)(at + lay.path_bytes);
+            double *sig64 = (double *)(at + 2 * lay.path_bytes);
+            double *grad64 = (double *)(at + 2 * lay.path_bytes + lay.sig_bytes);
+            void *inner_ws = at + 2 * lay.path_bytes + 2 * lay.sig_bytes;
+            const int64_t points = B * L * d, coefficients = rows * plan.sig_size;
+            hipLaunchKernelGGL(widen_kernel, dim3(convert_blocks(points)), dim3(256), 0, st, (const float *)path, path64,
+                               points);
+            const bool have_sig = sig && grad_sig && coefficients > 0;
+            if (have_sig)
+                hipLaunchKernelGGL(widen_kernel, dim3(convert_blocks(coefficients)), dim3(256), 0, st,
+                                   (const float *)grad_sig, grad64, coefficients);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return launch_failed(e, "conversion launch");
+            if (have_sig) {
+                rc = sig_forward_t<double>(path64, sig64, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows,
+                                           W, nullptr, 0, inner_ws, inner, st);
+                if (rc != PATHSIG_OK) return rc;
+            }
+            rc = sig_backward_t<double>(path64, have_sig ? sig64 : nullptr, have_sig ? grad64 : nullptr, gpath64, B, L, d,
+                                        depth, level_sizes, encoded_words, n_encoded, windows, W, nullptr, 0, inner_ws,
+                                        inner, st);
+            if (rc != PATHSIG_OK) return rc;
+            hipLaunchKernelGGL(narrow_kernel, dim3(convert_blocks(points)), dim3(256), 0, st, (const double *)gpath64,
+                               (float *)grad_path, points);
+            e = hipGetLastError();
+            if (e != hipSuccess) return launch_failed(e, "conversion launch");
+            return PATHSIG_OK;
         }
     }
     if (dtype == PATHSIG_F32)

@@ -51,6 +51,8 @@ struct Options {
     int64_t embed_share;     // a projection runs on the register-tiled kernels when its top level keeps at least
                              // 1/embed_share of the dense one (0: never; -1: the library's own rule)
     int64_t tiled;           // 0: every call takes the per-word kernels, whatever its shape (default 1)
+    int64_t deep_fp64;       // 1 (default): fp32 backward calls of depth 9 and more run their sweep in fp64 (see
+                             // backward_in_fp64 in api.hip); 0: in fp32 like every other call
 };
 const Options &options();
 

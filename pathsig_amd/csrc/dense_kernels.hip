@@ -800,15 +800,25 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
                 else
                     StepTargets<T, D, P, N, false, BOUND>::template run<G::kFwdSub, KS>(a, sub, dxs, dxs, dxp);
             };
-            read(0, dxs0, dxp0, dxf0);
-            int tt = 0;
-            for (; tt + 1 < nt; tt += 2) {
-                read(tt + 1, dxs1, dxp1, dxf1);
-                step(dxs0, dxp0, dxf0);
-                read(tt + 2 < nt ? tt + 2 : tt + 1, dxs0, dxp0, dxf0);
-                step(dxs1, dxp1, dxf1);
+            // (one set where two would not fit the register file beside the lane's state: fp64 over the widest
+            // alphabets, whose sweep otherwise keeps part of its state in scratch memory)
+            constexpr bool kTwoSets = sizeof(T) == 4 || 2 * (G::kFwdSub + 2 * (KS * D + FQ * FK + P)) <= 384;
+            if constexpr (kTwoSets) {
+                read(0, dxs0, dxp0, dxf0);
+                int tt = 0;
+                for (; tt + 1 < nt; tt += 2) {
+                    read(tt + 1, dxs1, dxp1, dxf1);
+                    step(dxs0, dxp0, dxf0);
+                    read(tt + 2 < nt ? tt + 2 : tt + 1, dxs0, dxp0, dxf0);
+                    step(dxs1, dxp1, dxf1);
+                }
+                if (tt < nt) step(dxs0, dxp0, dxf0);
+            } else {
+                for (int tt = 0; tt < nt; ++tt) {
+                    read(tt, dxs0, dxp0, dxf0);
+                    step(dxs0, dxp0, dxf0);
+                }
             }
-            if (tt < nt) step(dxs0, dxp0, dxf0);
         }
     }
     if constexpr (N - 1 >= P) {
@@ -1339,7 +1349,13 @@ struct BackwardShape {
         kSlab ? (kRowBytes * 32 <= 8192 ? 32 : kRowBytes * 16 <= 8192 ? 16 : 8)
               : (kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32
                  : kRowBytes * 16 <= 131072 ? 16 : kRowBytes * 8 <= 131072 ? 8 : 4);
-    static constexpr int kStage = kBwdTile * KS * D;
+    // Increments are staged for several tiles at a time where that takes little LDS (at most 4 KB, plus the
+    // increment of the ghost step; eight one-wave blocks with their slabs still share a CU): a round trip to
+    // memory per stage instead of one per tile.
+    static constexpr int kTileStage = kBwdTile * KS * D;
+    static constexpr int kStageRoom = 4096 / (kTileStage * (int)sizeof(T));
+    static constexpr int kStageTiles = !kSlab || kStageRoom < 1 ? 1 : kStageRoom > 8 ? 8 : kStageRoom;
+    static constexpr int kStage = kStageTiles * kTileStage + (kStageTiles > 1 ? KS * D : 0);
     static constexpr int kSums = G::kWaves * kParts;
     static constexpr int kSumRow = kBwdTile * kLetters;
     // fp64: the chain's P terms reach their letters through LDS (a row of D cells per lane, letter-major so that
@@ -1359,7 +1375,7 @@ __device__ __forceinline__ void dense_backward_body(
     const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
     const int pu_unit,  // index of the thread within its unit (its prefix, unless the first level is split)
     const int tid,      // index of the thread within its block
-    T (&sdx)[BackwardShape<T, D, N, P>::kStage],
+    T (&sdx_all)[BackwardShape<T, D, N, P>::kStage],
     T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
     T (&cells)[BackwardShape<T, D, N, P>::kCells], T (&slab)[BackwardShape<T, D, N, P>::kSlabElems], T (&carry)[D]) {
     using G = Geometry<D, N, P, sizeof(T)>;
@@ -1410,6 +1426,33 @@ __device__ __forceinline__ void dense_backward_body(
     const T *x = path + (b * shape.L + span.start) * D;
     T *ginc = grad_inc + (b * (shape.L - 1) + span.start) * D;
     const T *grow = grad_sig + row * G::kSigSize;
+
+    // A chunk that writes the path gradient itself (kToPath) owns the points begin .. end - 1 of its row (the last
+    // chunk also the final point): dL/dx[t] = g[t-1] - g[t] with g the per-increment sums.  The sum of the last
+    // increment before the chunk, g[begin - 1], belongs to the chunk on the left; this chunk computes it again with
+    // one more step of its sweep (tile -1, the ghost step: the state after increment `begin` is exactly what that
+    // step needs), so every point has one writer, nothing is added in memory and the order of the sums is fixed.
+    const int64_t len = end - begin;
+    const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
+    const bool ghost = kToPath && len > 0 && begin > 0;
+    // Increments reach LDS a stage at a time: the tiles ti - ti % kStageTiles .. ti share one (the leftmost stage
+    // also holds the ghost step).  The loads of the first stage are the first ones the kernel issues, so the loads
+    // of the state and of the upstream gradient below stay in flight while its increments are written.
+    constexpr int kStageTiles = BS::kStageTiles;
+    int64_t staged_from = 0;  // first increment in `sdx_all`
+    auto stage_for = [&](int64_t ti) {
+        if (ti < 0) {
+            if (kStageTiles > 1) return;  // part of the leftmost stage
+            staged_from = begin - 1;
+            stage_increments<T, D, KS, G::kBlock>(sdx_all, x + staged_from * D, 1, tid);
+        } else if (ti == ntiles - 1 || (ti + 1) % kStageTiles == 0) {
+            const int64_t first_tile = ti - ti % kStageTiles;
+            const int64_t until = end < begin + (ti + 1) * kBwdTile ? end : begin + (ti + 1) * kBwdTile;
+            staged_from = begin + first_tile * kBwdTile - (kStageTiles > 1 && first_tile == 0 && ghost ? 1 : 0);
+            stage_increments<T, D, KS, G::kBlock>(sdx_all, x + staged_from * D, (int)(until - staged_from), tid);
+        }
+    };
+    if (ntiles > 0) stage_for(ntiles - 1);
 
     // A: signature at the right edge of the unit (levels < N).  H: adjoint at the right edge.
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
@@ -1473,20 +1516,12 @@ __device__ __forceinline__ void dense_backward_body(
     }
 
 
-    const int64_t len = end - begin;
-    const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
-    // A chunk that writes the path gradient itself (kToPath) owns the points begin .. end - 1 of its row (the last
-    // chunk also the final point): dL/dx[t] = g[t-1] - g[t] with g the per-increment sums.  The sum of the last
-    // increment before the chunk, g[begin - 1], belongs to the chunk on the left; this chunk computes it again with
-    // one more step of its sweep (tile -1, the ghost step: the state after increment `begin` is exactly what that
-    // step needs), so every point has one writer, nothing is added in memory and the order of the sums is fixed.
-    const bool ghost = kToPath && len > 0 && begin > 0;
     for (int64_t ti = ntiles - 1; ti >= (ghost ? -1 : 0); --ti) {
         const int64_t t0 = ti < 0 ? begin - 1 : begin + ti * kBwdTile;
         const int nt = ti < 0 ? 1 : (int)((end - t0) < kBwdTile ? (end - t0) : kBwdTile);
-        const T *xw = x + t0 * D;
         lds_barrier();
-        stage_increments<T, D, KS, G::kBlock>(sdx, xw, nt, tid);
+        if (ti < ntiles - 1) stage_for(ti);
+        const T *sdx = sdx_all + (t0 - staged_from) * (KS * D);
         lds_barrier();
         auto step = [&](int tt, const T (&dxs)[KS][D], const T (&dxp)[P], const T (&dxf)[FQ][FK]) {
             // A_t = A_{t+1} (x) exp(-dx_t), levels < N

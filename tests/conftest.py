@@ -12,7 +12,8 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
-_OPTION_DEFAULTS = {"chunks": 0, "letter_bounds": 1, "logsig_scatter": 0, "batch_tile": 0, "embed_share": -1, "tiled": 1}
+_OPTION_DEFAULTS = {"chunks": 0, "letter_bounds": 1, "logsig_scatter": 0, "batch_tile": 0, "embed_share": -1, "tiled": 1,
+                    "deep_fp64": 1}
 
 
 @pytest.fixture

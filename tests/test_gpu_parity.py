@@ -19,15 +19,6 @@ TOL = {torch.float64: 1e-12, torch.float32: 1e-5}
 DEV = "cuda"
 
 
-def _grad_tol(dtype, depth):
-    """Gradient bound of the shapes that are swept in one piece.  The reverse sweep rebuilds the signature of
-    every earlier time by multiplying with exp(-dx_t); at depth 9 and more, over a span of increments of size one,
-    that loses digits in fp32 (1.0e-5 to 1.5e-5 of the largest gradient, tiled and per-word kernels alike; shapes that
-    are cut into time chunks take four chunks at least there and stay below 1e-5).  The reference's own suite allows
-    1e-4 below depth 10 and 1e-3 from there on for fp32 gradients (`tests/test_sig.py:26-34`)."""
-    return 3e-5 if (dtype == torch.float32 and depth >= 9) else TOL[dtype]
-
-
 @pytest.fixture(scope="module")
 def ps():
     import pathsig_amd
@@ -990,7 +981,7 @@ def test_shapes_whose_units_take_several_blocks(ps, dtype, d, depth):
         G = randn(tuple(want.shape), seed=501)
         got, grad = _run_sig(ps, path, depth, dtype, windows=windows, G=G)
         assert rel_err(got, want) < TOL[dtype]
-        assert rel_err(grad, TO.signature_vjp(path, G, depth, None, None, windows)) < _grad_tol(dtype, depth)
+        assert rel_err(grad, TO.signature_vjp(path, G, depth, None, None, windows)) < TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -1002,7 +993,7 @@ def test_largest_compiled_shapes(ps, dtype, d, depth):
     G = randn(tuple(want.shape), seed=701)
     got, grad = _run_sig(ps, path, depth, dtype, G=G)
     assert rel_err(got, want) < TOL[dtype]
-    assert rel_err(grad, TO.signature_vjp(path, G, depth)) < _grad_tol(dtype, depth)
+    assert rel_err(grad, TO.signature_vjp(path, G, depth)) < TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
@@ -1079,6 +1070,25 @@ def test_projection_and_windows_through_split_children(ps, dtype, d, depth, B):
             g2 = torch.ops.pathsig.signature_backward(x, sig, G.to(dtype).to(DEV), *args)
         assert torch.equal(sig, out.detach())
         assert rel_err(g2.cpu()[idx], want_grad) < TOL[dtype]
+
+
+@pytest.mark.parametrize("d,depth,windows", [(2, 12, None), (3, 10, [(0, 8), (2, 7), (3, 4)]), (4, 9, None)])
+def test_deep_fp32_backward_runs_in_fp64_unless_switched_off(ps, set_option, d, depth, windows):
+    """Option "deep_fp64": from depth 9 on an fp32 backward sweeps in fp64 and holds 1e-5 over increments of size
+    one; switched off it is the plain fp32 sweep, within the 1e-4 the reference's own suite allows there
+    (`tests/test_sig.py:26-34`), and the two differ."""
+    path = brownian_path(2, 8, d, seed=900 + d) * 2.0
+    want = TO.compute_signature(path, depth, None, None, windows)
+    G = randn(tuple(want.shape), seed=901)
+    want_grad = TO.signature_vjp(path, G, depth, None, None, windows)
+    grads = {}
+    for on in (1, 0):
+        set_option("deep_fp64", on)
+        got, grads[on] = _run_sig(ps, path, depth, torch.float32, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[torch.float32]
+    assert rel_err(grads[1], want_grad) < TOL[torch.float32]
+    assert rel_err(grads[0], want_grad) < 1e-4
+    assert not torch.equal(grads[0], grads[1])
 
 
 @pytest.mark.parametrize("d,depth,B", [(100, 3, 2), (8, 8, 1), (8, 8, 16)])

@@ -84,10 +84,11 @@ def test_random_signature_cases(set_option, seed):
         except RuntimeError:  # every window degenerate: the checker's output does not depend on the path
             want_grad = torch.zeros_like(path)
         tol = 1e-5 if dtype == torch.float32 else 1e-12
-        # at depth 10 and more the gradient of a top-level coefficient sums thousands of terms of mixed sign and
-        # fp32 rounding alone passes 1e-5 of the largest gradient: seed 15, case 29 (d = 2, depth 11, windows)
-        # gives 1.04e-5 here and 1.67e-5 in the literal fp32 restatement of the reference's kernel on the CPU
-        tol_grad = 3e-5 if (dtype == torch.float32 and depth >= 10) else tol
+        # (at depth 10 and more the gradient of a top-level coefficient sums thousands of terms of mixed sign; in fp32
+        # arithmetic rounding alone passes 1e-5 of the largest gradient there: seed 15, case 29 (d = 2, depth 11,
+        # windows) gives 1.67e-5 in the literal fp32 restatement of the reference's kernel on the CPU.  The library
+        # runs such a backward in fp64.)
+        tol_grad = tol
         what = f"seed {seed} case {case}: d={d} depth={depth} B={B} L={L} {dtype} windows={windows} chunks={chunks}"
         x = path.to(dtype).to(DEV).requires_grad_(True)
         win = None if windows is None else torch.tensor(windows, dtype=torch.int64, device=DEV)

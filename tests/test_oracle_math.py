@@ -278,6 +278,59 @@ def test_words_logsig_matches_tensor_logsig(d, depth, top):
     assert (gw - gt).abs().max() < 1e-12
 
 
+def _word_of(col, d, depth):
+    """Letters of the word at dense column `col` (levels one after the other, words in base-d order)."""
+    for n in range(1, depth + 1):
+        if col < d ** n:
+            return tuple((col // d ** (n - 1 - i)) % d for i in range(n))
+        col -= d ** n
+    raise AssertionError("column beyond the last level")
+
+
+def _power_by_cuts(logs, w, k):
+    """(L^(x)k)(w) from the definition: the sum over the ways to cut w into k non-empty consecutive pieces of the
+    product of L on the pieces."""
+    n, total = len(w), 0.0
+    for cuts in itertools.combinations(range(1, n), k - 1):
+        edges = (0,) + cuts + (n,)
+        term = 1.0
+        for a, b in zip(edges[:-1], edges[1:]):
+            term *= logs[w[a:b]]
+        total += term
+    return total
+
+
+@pytest.mark.parametrize("d,depth,top", [(2, 4, None), (3, 3, None), (3, 4, "lyndon"), (2, 5, "some")])
+def test_logsig_power_cache_against_powers_from_the_definition(d, depth, top):
+    """`logsig_power_cache` against tensor powers written out word by word (sums over the cuts of the word), of
+    a logarithm computed another way than the one the cache is usually built from (level by level from
+    exp(L) = S, not the alternating series)."""
+    from pathsig_amd.projections import lyndon_codes
+    path = randn((2, 5, d), seed=21) * 0.7
+    if top is None:
+        top_codes, top_size = None, d ** depth
+    elif top == "lyndon":
+        top_codes = lyndon_codes(d, depth)
+        top_size = len(top_codes)
+    else:
+        top_codes = [5, 0, 31, 12, 12, 7]
+        top_size = len(top_codes)
+    cols = TO.hybrid_columns(d, depth, top_size, top_codes)
+    dense_log = TO.logsignature(path, depth, method="inverse_exp")
+    got = TO.logsig_power_cache(dense_log[:, cols], depth, d, top_size, top_codes).reshape(2, len(cols), depth)
+    for row in range(2):
+        logs = {_word_of(c, d, depth): float(dense_log[row, c]) for c in range(dense_log.shape[1])}
+        for idx, col in enumerate(cols):
+            w = _word_of(col, d, depth)
+            powers = [_power_by_cuts(logs, w, k) for k in range(1, len(w) + 1)]
+            want = powers + [0.0] * (depth - len(w))
+            if len(w) < depth:
+                # the weight with which w enters the top-level sums of the adjoint as a prefix
+                want[len(w)] = -sum(powers[m - 1] / math.factorial(m + 1) for m in range(1, len(w) + 1))
+            for k in range(depth):
+                assert abs(float(got[row, idx, k]) - want[k]) < 1e-13, (row, w, k)
+
+
 # ------------------------------------------------------------------------------------------------
 # gradients
 # ------------------------------------------------------------------------------------------------
