@@ -244,8 +244,13 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
     if (rc != PATHSIG_OK) return rc;
     const DenseChoice dc = dense_choice(sizeof(T), d, depth, all_dense, level_sizes, B, L, shape.W, windows != nullptr);
     const size_t keep_need = dc.usable ? dc.keep_bytes : (size_t)(B * shape.W * plan.keep_size) * sizeof(T);
-    if (kept && (keep_need == 0 || kept_bytes < keep_need)) {
-        set_error("chunk buffer: this call keeps %zu bytes, got %zu", keep_need, kept_bytes);
+    // The layout of what a forward keeps follows from the choice of kernels, which the tuning switches can change
+    // between the two calls.  A buffer of another size than this call would have kept comes from a forward that
+    // chose differently and is refused (every such choice keeps a different number of bytes: prefix values per
+    // word, two rows of products per chunk, or the dense signature).
+    if (kept && (keep_need == 0 || kept_bytes != keep_need)) {
+        set_error("chunk buffer: the forward of this call keeps %zu bytes, got %zu (made under other options?)", keep_need,
+                  kept_bytes);
         return PATHSIG_ERR_ARGUMENT;
     }
     plan.keep = const_cast<void *>(kept);

@@ -1619,7 +1619,18 @@ __device__ __forceinline__ void dense_backward_body(
                     const int letter = base + row_letter<DP>(lane);
                     if (row_writer<DP>(lane) && letter < D) sg[wave * 4 + (lane >> 4)][tt * D + letter] = r;
                 }
+                // The passes below add to cells that other lanes of the same wave have just stored.  A wave's LDS
+                // operations complete in order; the fences keep the compiler from moving or merging them across
+                // the passes (no instruction is emitted for them).
+                auto order_wave_lds = [] {
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                };
+                // (the cells of a row of sixteen lanes belong to one wave, sg[wave * 4 + row]: a bounded sweep, which
+                // runs a copy of this body per wave, still has writer and adder in the same copy)
                 if constexpr (kLastDirect) {
+                    order_wave_lds();
                     // the term of the last prefix letter goes straight to its cell: the sixteen lanes of a row hold
                     // consecutive prefixes, so with sixteen letters or more their last letters differ
                     if (active) sg[wave * 4 + (lane >> 4)][tt * D + u[P - 1]] += gpre[P - 1];
@@ -1628,6 +1639,7 @@ __device__ __forceinline__ void dense_backward_body(
                         const T mine = with_first[j] ? gpre[j] : T(0);
                         const T sum_first = row_total(mine);
                         const T sum_last = row_total(gpre[j] - mine);
+                        order_wave_lds();
                         if ((lane & 15) == 0 && row_live) {
                             T *cells_of_step = &sg[wave * 4 + (lane >> 4)][tt * D];
                             cells_of_step[ua[j]] += sum_first;
@@ -1654,6 +1666,7 @@ __device__ __forceinline__ void dense_backward_body(
                     }
                     const T r = row_totals<T, KP>(padded, lane);
                     const int li = row_letter<KP>(lane);
+                    order_wave_lds();
                     if (row_writer<KP>(lane) && li < KF && a0 + li < D)
                         sg[wave * 4 + (lane >> 4)][tt * D + a0 + li] += r;
                 }

@@ -164,6 +164,9 @@ Tensor sig_backward(const Tensor &path_in, const Tensor &signature_in, const Ten
         TORCH_CHECK(chunks_in.is_cuda() && chunks_in.scalar_type() == path_in.scalar_type(),
                     "chunks must be a CUDA tensor of the path's dtype");
         chunks = chunks_in.contiguous();
+        // kept under other tuning switches than the ones in force now (its size tells): the backward recomputes
+        const size_t now = pathsig_sig_chunks_bytes(c.dt, c.B, c.L, c.d, (int)c.depth, c.sizes, c.W);
+        if ((size_t)chunks.numel() * chunks.element_size() != now) chunks = Tensor();
     }
     c10::DeviceGuard guard(c.path.device());
     Tensor out = at::empty_like(c.path);

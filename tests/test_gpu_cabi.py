@@ -87,6 +87,12 @@ def test_signature_entry_points(lib, dtype, case):
     stream.synchronize()
     if case == "dense_chunked":
         assert keep_bytes > 0
+        # a buffer of another size than this call keeps (one made under other tuning switches) is refused
+        for wrong in (keep_bytes - 256, keep_bytes + 256):
+            rc = lib.pathsig_sig_backward_kept(_p(x), _p(sig_k), _p(g), _p(grad_k), code, B, L, d, depth, host_sizes,
+                                               _p(words), n_words, _p(win), W, _p(keep), wrong, _p(bws), bws_bytes, handle)
+            assert rc != 0 and b"chunk buffer" in lib.pathsig_last_error()
+        stream.synchronize()
     assert rel_err(sig, want) < TOL[dtype] and rel_err(grad, want_grad) < TOL[dtype]
     assert torch.equal(sig_k, sig) and rel_err(grad_k, want_grad) < TOL[dtype]
 

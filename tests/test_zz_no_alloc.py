@@ -1,7 +1,8 @@
 """The signature backward that allocates nothing (`pathsig_sig_backward_noalloc`), called through the C ABI with
 raw device pointers, against `pathsig_sig_backward` with a caller-provided workspace: same inputs, two calls in a
 row (the second one smaller, so stale contents of the shared static scratch would show), fp32 1e-5 / fp64 1e-12
-with the metric of the other parity tests, plus the size limit."""
+with the metric of the other parity tests, plus the size limit, plus the two properties the entry point exists for:
+free device memory does not move across a call, and a call can be captured into a HIP graph and replayed."""
 from __future__ import annotations
 
 import ctypes
@@ -66,6 +67,57 @@ def test_noalloc_backward_matches_the_workspace_one(dtype):
         assert rc == 0, lib.pathsig_last_error()
         assert 0 < ws_bytes <= STATIC_BYTES
         assert torch.isfinite(got).all() and rel_err(got, want) < TOL[dtype], case
+
+
+def _call_pair(lib, path, sig, grad_sig, B, L, d, depth):
+    """(noalloc closure, workspace closure) on fixed device tensors; each returns the library's status code."""
+    got, want = torch.full_like(path, float("nan")), torch.full_like(path, float("nan"))
+    ws_bytes = lib.pathsig_sig_backward_workspace(0, B, L, d, depth, None, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+
+    def noalloc():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return lib.pathsig_sig_backward_noalloc(_p(path), _p(sig), _p(grad_sig), _p(got), 0, B, L, d, depth, None, None,
+                                                0, None, 0, stream)
+
+    def with_workspace():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return lib.pathsig_sig_backward(_p(path), _p(sig), _p(grad_sig), _p(want), 0, B, L, d, depth, None, None, 0,
+                                        None, 0, _p(ws), ws_bytes, stream)
+
+    return noalloc, with_workspace, got, want
+
+
+def test_noalloc_backward_leaves_free_memory_alone_and_can_be_captured():
+    import pathsig_amd as ps
+    from pathsig_amd import _load
+    lib = _load.lib()
+    B, L, d, depth = 6, 300, 4, 6
+    path = brownian_path(B, L, d, seed=11).float().to(DEV)
+    sig = ps.Signature(depth=depth)(path)
+    grad_sig = randn(tuple(sig.shape), seed=12).float().to(DEV)
+    noalloc, with_workspace, got, want = _call_pair(lib, path, sig, grad_sig, B, L, d, depth)
+    assert noalloc() == 0, lib.pathsig_last_error()     # warm-up: the scratch address is looked up once per device
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        assert noalloc() == 0, lib.pathsig_last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    # captured once, replayed on new inputs, with eager work and synchronisations between the replays
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = noalloc()
+    assert rc == 0, lib.pathsig_last_error()
+    for replay in range(3):
+        path.copy_(brownian_path(B, L, d, seed=20 + replay).float())
+        sig.copy_(ps.Signature(depth=depth)(path))
+        grad_sig.copy_(randn(tuple(sig.shape), seed=30 + replay).float())
+        got.fill_(float("nan"))
+        graph.replay()
+        assert with_workspace() == 0, lib.pathsig_last_error()
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all() and rel_err(got, want) < 1e-6, replay
 
 
 def test_noalloc_backward_rejects_what_does_not_fit():
