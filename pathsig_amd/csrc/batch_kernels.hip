@@ -8,7 +8,13 @@
 // of cells in LDS, [increment of the tile][letter][lane], updated with plain read-add-write (LDS float
 // atomics run at a small fraction of the plain LDS rate); the waves of a block share the G paths and
 // the staged increments, and after each tile the slabs are added up and flushed to the per-increment
-// gradient with one global atomic per (path, increment, letter) and block.  The arithmetic per word is
+// gradient with one global atomic per (path, increment, letter) and block.  (Two entries of a lane may carry the
+// same letter, so the read-add-writes of an increment form a chain, each waiting for the LDS round trip of the one
+// before.  Measured alternative: 64 paths to a group, so that a wave's letters are uniform and sit in scalar
+// registers, with the per-letter sums formed in sixteen vector registers indexed by those scalars and every cell
+// stored once: gfx950 has no relative register moves, the compiler brackets every indexed access with a switch
+// of the register-index mode, and the sweep of 2320 words over sixteen letters took 1077 us against 959 us.)
+// The arithmetic per word is
 // the same chain roll-back and chain adjoint as in words_kernels.hip
 // (reference: src/pathsig/backward/sig_backward_kernels.cu:120-342).
 #include <cstdlib>
@@ -312,9 +318,7 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
     hipError_t attr = hipSuccess;
 #define PSIG_LAUNCH(MAXDEG, GG)                                                                                    \
     do {                                                                                                           \
-        if (lds > 64 * 1024)                                                                                       \
-            attr = hipFuncSetAttribute((const void *)batch_backward_kernel<T, MAXDEG, GG, ACC>,                    \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                      \
+        if (lds > 64 * 1024) attr = allow_dynamic_lds<batch_backward_kernel<T, MAXDEG, GG, ACC>>(lds);             \
         if (attr != hipSuccess) return attr;                                                                       \
         hipLaunchKernelGGL((batch_backward_kernel<T, MAXDEG, GG, ACC>), grid, dim3(kBatchBlock), lds, stream, path, \
                            sig, grad_sig, grad_inc, shape, plan, codes, (int)tile);                                \

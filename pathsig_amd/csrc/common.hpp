@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "pathsig_hip.h"
 
 namespace psig {
@@ -102,6 +104,25 @@ __device__ __forceinline__ double wave_total(double v) {
     v = dpp_add_c<0x142, 0xA>(v);
     v = dpp_add_c<0x143, 0xC>(v);
     return v;
+}
+#endif
+
+#if defined(__HIPCC__)
+// A kernel that asks for more dynamic LDS than the default limit needs that limit raised first.  Done once per
+// kernel and device (the table belongs to the kernel: it is a template argument, not a function argument, since
+// kernels of one signature share a pointer type), and again only when a call asks for more than any before it.
+template <auto Kernel>
+hipError_t allow_dynamic_lds(size_t bytes) {
+    static std::atomic<size_t> allowed[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && allowed[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes);
+    if (e == hipSuccess && tracked) allowed[dev].store(bytes, std::memory_order_release);
+    return e;
 }
 #endif
 

@@ -676,8 +676,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
         const size_t top_bytes = (size_t)lp.top_dense * sizeof(T);
         if (rows >= 256 && top_bytes <= 64 * 1024) {
             if (top_bytes > 32 * 1024) {
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_top_rows_kernel<T>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)top_bytes);
+                e = allow_dynamic_lds<logsig_gather_top_rows_kernel<T>>(top_bytes);
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(blk), top_bytes, stream,
@@ -711,8 +710,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
         const bool a_in_lds = a_bytes <= 144 * 1024;
         if (a_in_lds) {
             if (a_bytes > 32 * 1024) {
-                e = hipFuncSetAttribute(reinterpret_cast<const void *>(logsig_gather_kernel<T, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)a_bytes);
+                e = allow_dynamic_lds<logsig_gather_kernel<T, true>>(a_bytes);
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL((logsig_gather_kernel<T, true>), dim3((unsigned)rows), dim3(blk), a_bytes, stream,
