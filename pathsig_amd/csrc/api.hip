@@ -370,6 +370,139 @@ DeepLayout deep_layout(int64_t B, int64_t L, int64_t d, int64_t rows, int64_t si
     return lay;
 }
 
+// Wide alphabets at depth 3.  The register-tiled kernels exist for every alphabet up to 64 letters; from 65 to 112
+// letters they exist for every eighth size (72, 80, .. 112).  A dense depth-3 call over d letters in that range
+// runs as the call over the next of these sizes D on a copy of the path with D - d constant coordinates: every
+// coefficient of a word that uses one of them is exactly zero, the others are the coefficients wanted, and the
+// gradient with respect to the added coordinates is dropped.  (The per-word kernels, which such calls took before,
+// run the backward of d = 100 at 0.4 TFLOP/s.)
+int64_t wide_pad_dim(size_t elem, int64_t d, int depth, bool all_dense, int64_t B, int64_t L, int64_t W, bool windowed) {
+    if (depth != 3 || !all_dense || d <= 64 || d > 112 || options().tiled == 0) return 0;
+    const int64_t D = (d + 7) / 8 * 8;
+    if (D == d) return 0;  // compiled as it is
+    return dense_choice(elem, D, depth, true, nullptr, B, L, W, windowed).usable ? D : 0;
+}
+
+// index of dense-layout column `col` of a depth-3 signature over d letters in the layout over D letters
+__device__ __forceinline__ int64_t wide_column(int64_t col, int64_t d, int64_t D) {
+    if (col < d) return col;
+    col -= d;
+    if (col < d * d) {
+        const int64_t a = col / d;
+        return D + a * D + (col - a * d);
+    }
+    col -= d * d;
+    const int64_t ab = col / d, c = col - ab * d, a = ab / d, b = ab - a * d;
+    return D + D * D + (a * D + b) * D + c;
+}
+
+// the first `count` values of every row: narrow[row][i] <-> wide[row][map(i)]; TO_WIDE copies narrow -> wide (the
+// rest of `wide` is cleared before where it is read), else wide -> narrow
+template <typename T, bool TO_WIDE, bool SIGNATURE>
+__global__ void __launch_bounds__(256) wide_copy_kernel(T *__restrict__ narrow, T *__restrict__ wide, int64_t rows,
+                                                        int64_t count, int64_t narrow_stride, int64_t wide_stride,
+                                                        int64_t d, int64_t D) {
+    const int64_t total = rows * count;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / count, col = i - row * count;
+        // a path row is one point: the letters keep their places; a signature row is mapped level by level
+        const int64_t at = row * wide_stride + (SIGNATURE ? wide_column(col, d, D) : col);
+        if (TO_WIDE) wide[at] = narrow[row * narrow_stride + col];
+        else narrow[row * narrow_stride + col] = wide[at];
+    }
+}
+
+template <typename T, bool TO_WIDE, bool SIGNATURE>
+hipError_t launch_wide_copy(const T *narrow, const T *wide, int64_t rows, int64_t count, int64_t narrow_stride,
+                            int64_t wide_stride, int64_t d, int64_t D, hipStream_t stream) {
+    if (rows * count == 0) return hipSuccess;
+    hipLaunchKernelGGL((wide_copy_kernel<T, TO_WIDE, SIGNATURE>), dim3(convert_blocks(rows * count)), dim3(256), 0, stream,
+                       const_cast<T *>(narrow), const_cast<T *>(wide), rows, count, narrow_stride, wide_stride, d, D);
+    return hipGetLastError();
+}
+
+struct WideLayout {
+    size_t path_bytes, sig_bytes;  // of the copies over D letters
+    int64_t sig_size, wide_sig_size;
+};
+WideLayout wide_layout(size_t elem, int64_t B, int64_t L, int64_t d, int64_t D, int64_t rows) {
+    WideLayout lay;
+    lay.sig_size = d + d * d + d * d * d;
+    lay.wide_sig_size = D + D * D + D * D * D;
+    lay.path_bytes = align_up((size_t)(B * L * D) * elem);
+    lay.sig_bytes = align_up((size_t)(rows * lay.wide_sig_size) * elem);
+    return lay;
+}
+
+template <typename T>
+int wide_forward(const void *path, void *sig, int64_t B, int64_t L, int64_t d, int64_t D, const int32_t *windows,
+                 int64_t W, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    const int64_t rows = B * (windows ? W : 1);
+    const WideLayout lay = wide_layout(sizeof(T), B, L, d, D, rows);
+    const size_t inner = pathsig_sig_forward_workspace(sizeof(T) == 8 ? PATHSIG_F64 : PATHSIG_F32, B, L, D, 3, nullptr,
+                                                       windows ? W : 0);
+    const size_t need = lay.path_bytes + lay.sig_bytes + inner;
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    unsigned char *at = (unsigned char *)workspace;
+    T *wide_path = (T *)at, *wide_sig = (T *)(at + lay.path_bytes);
+    hipError_t e = launch_fill_zero<T>(wide_path, B * L * D, stream);
+    if (e == hipSuccess) e = launch_wide_copy<T, true, false>((const T *)path, wide_path, B * L, d, d, D, d, D, stream);
+    if (e != hipSuccess) return launch_failed(e, "wide path launch");
+    const int rc = sig_forward_t<T>(wide_path, wide_sig, B, L, D, 3, nullptr, nullptr, 0, windows, W, nullptr, 0,
+                                    at + lay.path_bytes + lay.sig_bytes, inner, stream);
+    if (rc != PATHSIG_OK) return rc;
+    e = launch_wide_copy<T, false, true>((const T *)sig, wide_sig, rows, lay.sig_size, lay.sig_size, lay.wide_sig_size, d,
+                                         D, stream);
+    if (e != hipSuccess) return launch_failed(e, "wide gather launch");
+    return PATHSIG_OK;
+}
+
+size_t wide_backward_bytes(size_t elem, int64_t B, int64_t L, int64_t d, int64_t D, int64_t W) {
+    const WideLayout lay = wide_layout(elem, B, L, d, D, B * (W > 0 ? W : 1));
+    return 2 * lay.path_bytes + 2 * lay.sig_bytes +
+           pathsig_sig_backward_workspace(elem == 8 ? PATHSIG_F64 : PATHSIG_F32, B, L, D, 3, nullptr, W);
+}
+
+template <typename T>
+int wide_backward(const void *path, const void *sig, const void *grad_sig, void *grad_path, int64_t B, int64_t L,
+                  int64_t d, int64_t D, const int32_t *windows, int64_t W, void *workspace, size_t workspace_bytes,
+                  hipStream_t stream) {
+    const int64_t rows = B * (windows ? W : 1);
+    const WideLayout lay = wide_layout(sizeof(T), B, L, d, D, rows);
+    const size_t need = wide_backward_bytes(sizeof(T), B, L, d, D, windows ? W : 0);
+    if (!workspace || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return PATHSIG_ERR_WORKSPACE;
+    }
+    unsigned char *at = (unsigned char *)workspace;
+    T *wide_path = (T *)at, *wide_gpath = (T *)(at + lay.path_bytes);
+    T *wide_sig = (T *)(at + 2 * lay.path_bytes), *wide_grad = (T *)(at + 2 * lay.path_bytes + lay.sig_bytes);
+    void *inner_ws = at + 2 * lay.path_bytes + 2 * lay.sig_bytes;
+    // (the coefficients of the words that use an added letter are zero in the signature, and their upstream
+    // gradient is taken as zero: they are no outputs of the call)
+    // Of the signature the reverse sweep reads the levels below the top one (its state at the right end): the first
+    // two levels are copied into a cleared buffer.
+    hipError_t e = launch_fill_zero<T>(wide_path, B * L * D, stream);
+    if (e == hipSuccess) e = launch_fill_zero<T>(wide_sig, 2 * (int64_t)(lay.sig_bytes / sizeof(T)), stream);
+    if (e == hipSuccess) e = launch_wide_copy<T, true, false>((const T *)path, wide_path, B * L, d, d, D, d, D, stream);
+    if (e == hipSuccess)
+        e = launch_wide_copy<T, true, true>((const T *)sig, wide_sig, rows, d + d * d, lay.sig_size, lay.wide_sig_size, d,
+                                            D, stream);
+    if (e == hipSuccess)
+        e = launch_wide_copy<T, true, true>((const T *)grad_sig, wide_grad, rows, lay.sig_size, lay.sig_size,
+                                            lay.wide_sig_size, d, D, stream);
+    if (e != hipSuccess) return launch_failed(e, "wide scatter launch");
+    const int rc = sig_backward_t<T>(wide_path, wide_sig, wide_grad, wide_gpath, B, L, D, 3, nullptr, nullptr, 0, windows, W,
+                                     nullptr, 0, inner_ws, need - 2 * lay.path_bytes - 2 * lay.sig_bytes, stream);
+    if (rc != PATHSIG_OK) return rc;
+    e = launch_wide_copy<T, false, false>((const T *)grad_path, wide_gpath, B * L, d, d, D, d, D, stream);
+    if (e != hipSuccess) return launch_failed(e, "wide gradient launch");
+    return PATHSIG_OK;
+}
+
 int check_logsig(int dtype, int64_t rows, int64_t d, int depth, int64_t top_size) {
     if (dtype != PATHSIG_F32 && dtype != PATHSIG_F64) {
         set_error("dtype must be PATHSIG_F32 or PATHSIG_F64 (got %d)", dtype);
@@ -449,6 +582,10 @@ size_t pathsig_sig_forward_workspace(int dtype, int64_t B, int64_t L, int64_t d,
     LevelPlan plan;
     bool all_dense;
     if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
+    if (const int64_t D = wide_pad_dim(elem_size(dtype), d, depth, all_dense, B, L, W > 0 ? W : 1, W > 0)) {
+        const WideLayout lay = wide_layout(elem_size(dtype), B, L, d, D, B * (W > 0 ? W : 1));
+        return lay.path_bytes + lay.sig_bytes + pathsig_sig_forward_workspace(dtype, B, L, D, depth, nullptr, W);
+    }
     const DenseChoice dc =
         dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
     return dc.usable ? dc.forward_workspace : 0;
@@ -487,6 +624,23 @@ int pathsig_sig_forward_keep(const void *path, void *sig, int dtype, int64_t B, 
         set_error("W must be >= 0");
         return PATHSIG_ERR_ARGUMENT;
     }
+    if (depth == 3 && d > 64 && B > 0 && (!windows || W > 0)) {
+        LevelPlan plan;
+        bool all_dense;
+        rc = build_plan(d, depth, level_sizes, n_encoded, encoded_words != nullptr, &plan, &all_dense);
+        if (rc != PATHSIG_OK) return rc;
+        if (const int64_t D = wide_pad_dim(elem_size(dtype), d, depth, all_dense, B, L, windows ? W : 1, windows != nullptr)) {
+            if (chunks && chunks_bytes > 0) {
+                set_error("chunk buffer: this call keeps 0 bytes, got %zu", chunks_bytes);
+                return PATHSIG_ERR_ARGUMENT;
+            }
+            if (dtype == PATHSIG_F32)
+                return wide_forward<float>(path, sig, B, L, d, D, windows, W, workspace, workspace_bytes,
+                                           (hipStream_t)stream);
+            return wide_forward<double>(path, sig, B, L, d, D, windows, W, workspace, workspace_bytes,
+                                        (hipStream_t)stream);
+        }
+    }
     if (dtype == PATHSIG_F32)
         return sig_forward_t<float>(path, sig, B, L, d, depth, level_sizes, encoded_words, n_encoded, windows, W,
                                     chunks, chunks_bytes, workspace, workspace_bytes, (hipStream_t)stream);
@@ -502,6 +656,8 @@ size_t pathsig_sig_backward_workspace(int dtype, int64_t B, int64_t L, int64_t d
     if (build_plan(d, depth, level_sizes, INT64_MAX, true, &plan, &all_dense) != PATHSIG_OK) return 0;
     const DenseChoice dc =
         dense_choice(elem_size(dtype), d, depth, all_dense, level_sizes, B, L, W > 0 ? W : 1, W > 0);
+    if (const int64_t D = wide_pad_dim(elem_size(dtype), d, depth, all_dense, B, L, W > 0 ? W : 1, W > 0))
+        return wide_backward_bytes(elem_size(dtype), B, L, d, D, W);
     if (backward_in_fp64(dtype, depth, dc)) {
         const size_t inner = std::max(pathsig_sig_backward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, W),
                                       pathsig_sig_forward_workspace(PATHSIG_F64, B, L, d, depth, level_sizes, W));
@@ -589,6 +745,23 @@ int pathsig_sig_backward_kept(const void *path, const void *sig, const void *gra
         if (!empty) {
             set_error("sig and grad_sig must not be NULL");
             return PATHSIG_ERR_ARGUMENT;
+        }
+    }
+    if (depth == 3 && d > 64 && B > 0 && (!windows || W > 0) && sig && grad_sig) {
+        LevelPlan plan;
+        bool all_dense;
+        rc = build_plan(d, depth, level_sizes, n_encoded, encoded_words != nullptr, &plan, &all_dense);
+        if (rc != PATHSIG_OK) return rc;
+        if (const int64_t D = wide_pad_dim(elem_size(dtype), d, depth, all_dense, B, L, windows ? W : 1, windows != nullptr)) {
+            if (chunks && chunks_bytes > 0) {
+                set_error("chunk buffer: the forward of this call keeps 0 bytes, got %zu", chunks_bytes);
+                return PATHSIG_ERR_ARGUMENT;
+            }
+            if (dtype == PATHSIG_F32)
+                return wide_backward<float>(path, sig, grad_sig, grad_path, B, L, d, D, windows, W, workspace,
+                                            workspace_bytes, (hipStream_t)stream);
+            return wide_backward<double>(path, sig, grad_sig, grad_path, B, L, d, D, windows, W, workspace,
+                                         workspace_bytes, (hipStream_t)stream);
         }
     }
     if (dtype == PATHSIG_F32 && depth >= 9 && B > 0) {

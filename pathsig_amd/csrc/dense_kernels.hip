@@ -802,7 +802,9 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             };
             // (one set where two would not fit the register file beside the lane's state: fp64 over the widest
             // alphabets, whose sweep otherwise keeps part of its state in scratch memory)
-            constexpr bool kTwoSets = sizeof(T) == 4 || 2 * (G::kFwdSub + 2 * (KS * D + FQ * FK + P)) <= 384;
+            // (nor beside the hundred and more children of a lane over the widest alphabets)
+            constexpr bool kTwoSets = (sizeof(T) == 4 && D <= 64) ||
+                                      (sizeof(T) == 8 && 2 * (G::kFwdSub + 2 * (KS * D + FQ * FK + P)) <= 384);
             if constexpr (kTwoSets) {
                 read(0, dxs0, dxp0, dxf0);
                 int tt = 0;
@@ -1686,7 +1688,7 @@ __device__ __forceinline__ void dense_backward_body(
                 }
             }
         };
-        if constexpr (sizeof(T) == 4) {
+        if constexpr (sizeof(T) == 4 && D <= 64) {
             // two register sets of increments, so the LDS reads of the next step hide behind the current one
             T dxs0[KS][D], dxp0[P], dxs1[KS][D], dxp1[P];
             T dxf0[FQ][FK], dxf1[FQ][FK];
@@ -1704,7 +1706,7 @@ __device__ __forceinline__ void dense_backward_body(
             }
             if (tt == 0) step(0, dxs0, dxp0, dxf0);
         } else {
-            // fp64 state fills the register file: one set of increments
+            // fp64 state, or a hundred children and their adjoints, fill the register file: one set of increments
             for (int tt = nt - 1; tt >= 0; --tt) {
                 T dxs[KS][D], dxp[P];
                 T dxf[FQ][FK];
@@ -1879,7 +1881,9 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
     X(253, 36, 3, 2, 2, 1) X(254, 37, 3, 2, 2, 1) X(255, 38, 3, 2, 2, 1) X(256, 39, 3, 2, 2, 1) \
     X(257, 40, 3, 2, 2, 1) X(258, 41, 3, 2, 2, 1) X(259, 42, 3, 2, 2, 1) X(260, 43, 3, 2, 2, 1) \
     X(261, 44, 3, 2, 2, 1) X(262, 45, 3, 2, 2, 1) X(263, 46, 3, 2, 2, 1) X(264, 47, 3, 2, 2, 1) \
-    X(265, 48, 3, 2, 2, 1)
+    X(265, 48, 3, 2, 2, 1) \
+    X(266, 80, 3, 2, 2, 1) X(267, 96, 3, 2, 2, 1) X(268, 112, 3, 2, 2, 1) X(269, 72, 3, 2, 2, 1) \
+    X(270, 88, 3, 2, 2, 1) X(271, 104, 3, 2, 2, 1)
 
 // The scan kernel of the time-chunked backward streams rows of levels 1..N-1 through a double buffer and keeps
 // two result rows, all in LDS; a shape whose rows are too long for that in type T is swept unchunked in T.

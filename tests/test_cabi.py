@@ -83,10 +83,16 @@ def test_argument_errors_have_codes_and_messages(lib):
 
 def test_workspace_sizes(lib):
     # general kernels: the forward needs none, the backward one increment accumulator
-    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 65, 3, None, 0) == 0
-    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 65, 3, None, 0)
-    assert need >= 4 * 99 * 65 * 4
-    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 65, 3, None, 0) >= 4 * 99 * 65 * 8
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 120, 3, None, 0) == 0
+    need = lib.pathsig_sig_backward_workspace(0, 4, 100, 120, 3, None, 0)
+    assert need >= 4 * 99 * 120 * 4
+    assert lib.pathsig_sig_backward_workspace(1, 4, 100, 120, 3, None, 0) >= 4 * 99 * 120 * 8
+    # 65 letters at depth 3 run as 72 letters on copies: of the path and the signature in the forward, of the path
+    # (twice), the signature and its gradient in the backward
+    wide_sig, wide_path = 4 * (72 + 72 ** 2 + 72 ** 3) * 4, 4 * 100 * 72 * 4
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 65, 3, None, 0) >= wide_sig + wide_path
+    assert lib.pathsig_sig_backward_workspace(0, 4, 100, 65, 3, None, 0) >= 2 * wide_sig + 2 * wide_path
+    assert lib.pathsig_sig_forward_workspace(0, 4, 100, 72, 3, None, 0) == 0     # compiled as it is, one piece
     # a long path on a tiled shape is cut into chunks, which need scratch in the forward too
     assert lib.pathsig_sig_forward_workspace(0, 128, 1024, 4, 6, None, 0) > 0
     assert lib.pathsig_sig_forward_workspace(0, 4096, 64, 4, 6, None, 0) == 0

@@ -26,6 +26,7 @@ def _compiled_shapes():
     shapes = [(d, n) for d in range(2, 9) for n in range(2, 8)]
     shapes += [(d, n) for d in range(9, 13) for n in range(2, 7)] + [(d, n) for d in range(13, 17) for n in range(2, 6)]
     shapes += [(d, n) for d in range(17, 33) for n in range(2, 5)] + [(d, n) for d in range(33, 65) for n in (2, 3)]
+    shapes += [(72, 3), (80, 3), (88, 3), (96, 3), (104, 3), (112, 3)]
     shapes += [(2, 8), (2, 9), (2, 10), (2, 11), (2, 12), (3, 8), (3, 9), (3, 10), (3, 11), (3, 12), (4, 8), (4, 9), (4, 10),
                (4, 11), (5, 8), (5, 9), (6, 8), (7, 8)]
     return shapes
@@ -35,7 +36,7 @@ def _compiled_shapes():
 def test_tiled_and_per_word_kernels_agree_on_every_compiled_shape(set_option, part):
     import pathsig_amd as ps
     shapes = _compiled_shapes()
-    assert len(shapes) == 208
+    assert len(shapes) == 214
     rng = random.Random(100 + part)
     for d, n in shapes[part::8]:
         size = sum(d ** k for k in range(1, n + 1))
@@ -119,7 +120,28 @@ def test_every_compiled_shape_against_the_oracle(part):
             torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("d", [65, 100])
+@pytest.mark.parametrize("d", [65, 79, 81, 100, 111])
 def test_widest_alphabets_of_the_reference_sweep_against_the_oracle(d):
+    """Alphabets between the compiled sizes 64, 72, 80, .. 112 run as the next compiled size on a path with constant
+    extra coordinates."""
     import pathsig_amd as ps
     _against_oracle(ps, d, 3, 2, 10, 77 + d, [0, 1], f"d={d} depth=3 B=2 L=10")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_padded_wide_alphabet_with_windows_and_both_kernel_families(set_option, dtype):
+    import pathsig_amd as ps
+    d, B, L = 70, 3, 12
+    path = brownian_path(B, L, d, seed=41)
+    windows = [(0, 12), (2, 9), (5, 6), (7, 7)]
+    want = TO.compute_signature(path, 3, None, None, windows)
+    G = randn(tuple(want.shape), seed=42)
+    want_grad = TO.signature_vjp(path, G, 3, None, None, windows)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    win = torch.tensor(windows, dtype=torch.int64, device=DEV)
+    for tiled in (1, 0):
+        set_option("tiled", tiled)
+        x = path.to(dtype).to(DEV).requires_grad_(True)
+        out = ps.Signature(depth=3, windows=win)(x)
+        (grad,) = torch.autograd.grad(out, x, G.to(dtype).to(DEV))
+        assert rel_err(out, want) < tol and rel_err(grad, want_grad) < tol, tiled
