@@ -1191,8 +1191,10 @@ struct EdgesShape {
     static constexpr size_t kStaticBytes = 2 * kRowBytes;  // the double buffer of the scans
     static constexpr size_t kCombineBytes = CombineShape<T, D, N, PC, kCombineBlock>::kBytes;  // staging of the combine
     static constexpr size_t kBudget = 78 * 1024;           // two blocks to a CU
-    static constexpr bool kUsable = kThreads <= 512 && GC::kBlock % kCombineBlock == 0 && N >= 2 && !GS::kOnePiece &&
-                                    kRowBytes % 16 == 0 && kStaticBytes + kCombineBytes <= kBudget;
+    // (compiled for fp32 from depth 4 on: the launch it saves matters where a step takes a hundred microseconds,
+    // and every instantiation adds to the library)
+    static constexpr bool kUsable = sizeof(T) == 4 && N >= 4 && kThreads <= 512 && GC::kBlock % kCombineBlock == 0 &&
+                                    !GS::kOnePiece && kRowBytes % 16 == 0 && kStaticBytes + kCombineBytes <= kBudget;
 };
 
 template <typename T, int D, int N, int P, bool ascending>
