@@ -454,14 +454,39 @@ template <typename T, int D>
 __device__ __forceinline__ constexpr int inc_slot(int a) { return (D % 4 == 0 && sizeof(T) == 4) ? (a ^ 1) : a; }
 
 // Stages nt increments as sdx[(tt * KS + q) * D + inc_slot(a)] = (x[tt+1][a] - x[tt][a]) / (q + 1).
+// (the loads of four rounds are issued before the first of them is waited for: the points come from memory, and a
+// chunk of 64 increments over four letters is four rounds of a wave)
 template <typename T, int D, int KS, int BLOCK>
 __device__ __forceinline__ void stage_increments(T *sdx, const T *__restrict__ xw, int nt, int tid) {
-    for (int idx = tid; idx < nt * D; idx += BLOCK) {
-        const T inc = xw[idx + D] - xw[idx];
-        const int tt = idx / D, a = idx - tt * D;
+    constexpr int kRounds = 4;
+    const int count = nt * D;
+    for (int first = 0; first < count; first += kRounds * BLOCK) {
+        T later[kRounds], earlier[kRounds];
 #pragma unroll
-        for (int q = 0; q < KS; ++q) sdx[(tt * KS + q) * D + inc_slot<T, D>(a)] = inc * rcp<T>(q + 1);
+        for (int i = 0; i < kRounds; ++i) {
+            // (an index beyond the end reads the last element again: loads under a condition would be branches,
+            // and a load the compiler cannot see consumed on every path is waited for at its register's next
+            // use, together with every store issued since)
+            const int idx = first + i * BLOCK + tid;
+            const int at = idx < count ? idx : count - 1;
+            later[i] = xw[at + D];
+            earlier[i] = xw[at];
+        }
+#pragma unroll
+        for (int i = 0; i < kRounds; ++i) {
+            const int idx = first + i * BLOCK + tid;
+            if (idx < count) {
+                const T inc = later[i] - earlier[i];
+                const int tt = idx / D, a = idx - tt * D;
+#pragma unroll
+                for (int q = 0; q < KS; ++q) sdx[(tt * KS + q) * D + inc_slot<T, D>(a)] = inc * rcp<T>(q + 1);
+            }
+        }
     }
+    // Every load above has been consumed.  Saying so (s_waitcnt vmcnt(0), which waits for nothing here) keeps the
+    // compiler from waiting later, where it cannot tell any more and global stores are in flight that the wait
+    // would include.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
 template <typename T, int D, int P, int KS>
@@ -566,53 +591,95 @@ __device__ __forceinline__ void prefix_letters(int pu, int (&u)[P]) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Place of the elements of a dense-layout row that lives in LDS.
+// The lanes of a wave hold consecutive prefixes, so they touch such a row at addresses D^r elements apart (r = 1,
+// 2, ..): for an alphabet that is a power of two these strides are multiples of the 64 LDS banks from D^r = 64 on,
+// and all lanes of a 16-byte access meet in four banks (measured on (4, 6): a product of two chunk signatures
+// through LDS took 10 000 clocks for 500 multiply-adds per lane).  SKEW rows are therefore stored with four
+// elements of padding after every 64, counted from a shifted origin that puts the first element of every level of
+// 64 words and more on a multiple of 64: a run of D^r elements that starts at a multiple of D^r within its level
+// then lies in one piece (D^r <= 64) or starts a block of 64 (D^r > 64), so its elements keep offsets known at
+// compile time, and lanes 64 elements apart are four banks apart.
+// ---------------------------------------------------------------------------------------------
+template <int D, bool SKEW>
+struct RowPlace {
+    static constexpr bool kOn = SKEW && D % 4 == 0 && (D & (D - 1)) == 0 && D <= 64;
+    static constexpr int shift() {
+        if (!kOn) return 0;
+        int below = 0, w = D;  // words of the levels whose size is not a multiple of 64
+        while (w % 64 != 0) {
+            below += w;
+            w *= D;
+        }
+        return (64 - below % 64) % 64;
+    }
+    static constexpr int kShift = shift();
+    static __host__ __device__ constexpr int pos(int idx) {
+        if (!kOn) return idx;
+        const int j = idx + kShift;
+        return j + ((j >> 6) << 2);
+    }
+    // element iv of a run that starts at pos(first) with first a multiple of the run's length within its level
+    static __host__ __device__ constexpr int in_run(int iv) { return kOn ? iv + ((iv >> 6) << 2) : iv; }
+    // elements of LDS that a row of `count` elements takes
+    static constexpr int size(int count) { return kOn ? (pos(count - 1) + 4) / 4 * 4 : count; }
+};
+
+// ---------------------------------------------------------------------------------------------
 // lane state <-> dense layout in memory
 // ---------------------------------------------------------------------------------------------
 // Reads the chain a[1..P] and the sub-trie levels P+1..TOP of prefix pu from a dense-layout row.
 // K < D: the lane holds the children a0 .. a0 + K - 1 of its prefix only (those beyond the alphabet read as zero).
-template <typename T, int D, int P, int TOP, int SUB, int K = D>
+// SKEW: the row lives in LDS in the layout of RowPlace (whole sets of children only).
+template <typename T, int D, int P, int TOP, int SUB, int K = D, bool SKEW = false>
 __device__ __forceinline__ void load_state(const T *__restrict__ row, int pu, bool active, T (&a)[P + 1], T (&sub)[SUB],
                                            int a0 = 0) {
     using G = Geometry<D, TOP, P>;
+    using RP = RowPlace<D, SKEW>;
+    static_assert(!RP::kOn || K == D, "skewed rows hold whole sets of children");
     int rest = 1;
 #pragma unroll
     for (int j = P; j >= 1; --j) {
-        a[j] = active ? row[G::level_off(j) + pu / rest] : T(0);
+        a[j] = active ? row[RP::pos((int)G::level_off(j) + pu / rest)] : T(0);
         rest *= D;
     }
     static_for<1, TOP - P + 1>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         constexpr int below = ipow(D, k - 1);  // words of this level below one child
         constexpr int off = sub_size(D, K, k - 1);
-        const T *src = row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
+        const T *src = RP::kOn ? row + RP::pos((int)G::level_off(P + k) + pu * D * below)
+                               : row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
 #pragma unroll
         for (int i = 0; i < K * below; ++i) {
             const bool have = K == D || a0 + i / below < D;
-            sub[off + i] = (active && have) ? src[i] : T(0);
+            sub[off + i] = (active && have) ? src[RP::in_run(i)] : T(0);
         }
     });
 }
 
-template <typename T, int D, int P, int TOP, int SUB, int K = D>
+template <typename T, int D, int P, int TOP, int SUB, int K = D, bool SKEW = false>
 __device__ __forceinline__ void store_state(T *__restrict__ row, int pu, const T (&a)[P + 1], const T (&sub)[SUB],
                                             int a0 = 0) {
     using G = Geometry<D, TOP, P>;
+    using RP = RowPlace<D, SKEW>;
+    static_assert(!RP::kOn || K == D, "skewed rows hold whole sets of children");
     // Every lane writes its chain values: lanes that share a chain node computed it with the same
     // operations, so they store identical bits, and no branch is needed.
     int rest = 1;
 #pragma unroll
     for (int j = P; j >= 1; --j) {
-        row[G::level_off(j) + pu / rest] = a[j];
+        row[RP::pos((int)G::level_off(j) + pu / rest)] = a[j];
         rest *= D;
     }
     static_for<1, TOP - P + 1>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         constexpr int below = ipow(D, k - 1);
         constexpr int off = sub_size(D, K, k - 1);
-        T *dst = row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
+        T *dst = RP::kOn ? row + RP::pos((int)G::level_off(P + k) + pu * D * below)
+                         : row + G::level_off(P + k) + ((int64_t)pu * D + a0) * below;
 #pragma unroll
         for (int i = 0; i < K * below; ++i)
-            if (K == D || a0 + i / below < D) dst[i] = sub[off + i];
+            if (K == D || a0 + i / below < D) dst[RP::in_run(i)] = sub[off + i];
     });
 }
 
@@ -638,10 +705,11 @@ struct SubWords {
 //   (A (x) B)(u v) = sum_{k<=P} A(u_1..u_k) B(u_{k+1}..u_P v) + sum_{j<|v|} A(u v_1..v_j) B(v_{j+1}..) + A(u v)
 // Sub-trie levels go top-down and the chain last, so everything read is still the old A.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int P, int TOP, int SUB>
+template <typename T, int D, int P, int TOP, int SUB, bool SKEW = false>
 __device__ __forceinline__ void apply_right(T (&a)[P + 1], T (&sub)[SUB], const T *__restrict__ B,
                                             const SubWords<D, P> &sw) {
     using G = Geometry<D, TOP, P>;
+    using RP = RowPlace<D, SKEW>;
     a[0] = T(1);
     static_for<0, TOP - P>([&](auto rc) {
         constexpr int r = TOP - P - decltype(rc)::value;  // TOP-P .. 1
@@ -657,14 +725,15 @@ __device__ __forceinline__ void apply_right(T (&a)[P + 1], T (&sub)[SUB], const 
             constexpr int offj = trie_size(D, j - 1);
 #pragma unroll
             for (int iv = 0; iv < width; ++iv)
-                acc[iv] = fmad<T>(sub[offj + iv / tail], B[G::level_off(r - j) + iv % tail], acc[iv]);
+                acc[iv] = fmad<T>(sub[offj + iv / tail], B[RP::pos((int)G::level_off(r - j) + iv % tail)], acc[iv]);
         });
         // chain values times B at (suffix of the prefix) . v
         static_for<0, P + 1>([&](auto kc) {
             constexpr int k = decltype(kc)::value;
-            const T *run = B + G::level_off(P - k + r) + (int64_t)sw.code[k][P] * width;
+            const T *run = RP::kOn ? B + RP::pos((int)G::level_off(P - k + r) + sw.code[k][P] * width)
+                                   : B + G::level_off(P - k + r) + (int64_t)sw.code[k][P] * width;
 #pragma unroll
-            for (int iv = 0; iv < width; ++iv) acc[iv] = fmad<T>(a[k], run[iv], acc[iv]);
+            for (int iv = 0; iv < width; ++iv) acc[iv] = fmad<T>(a[k], run[RP::in_run(iv)], acc[iv]);
         });
 #pragma unroll
         for (int iv = 0; iv < width; ++iv) sub[off + iv] = acc[iv];
@@ -673,7 +742,7 @@ __device__ __forceinline__ void apply_right(T (&a)[P + 1], T (&sub)[SUB], const 
     for (int i = P; i >= 1; --i) {
         T acc = a[i];
 #pragma unroll
-        for (int k = 0; k < i; ++k) acc = fmad<T>(a[k], B[G::level_off(i - k) + sw.code[k][i]], acc);
+        for (int k = 0; k < i; ++k) acc = fmad<T>(a[k], B[RP::pos((int)G::level_off(i - k) + sw.code[k][i])], acc);
         a[i] = acc;
     }
 }
@@ -684,23 +753,26 @@ __device__ __forceinline__ void apply_right(T (&a)[P + 1], T (&sub)[SUB], const 
 // B is a dense-layout row with levels 1..N-1.  The chain goes first (ascending), then the sub-trie
 // levels top-down in depth, so everything read is still the old H.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int N, int P, int HSUB>
+template <typename T, int D, int N, int P, int HSUB, bool SKEW = false>
 __device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], const T *__restrict__ B,
                                                const SubWords<D, P> &sw) {
     using G = Geometry<D, N, P>;
+    using RP = RowPlace<D, SKEW>;
     constexpr int R = N - P;
 #pragma unroll
     for (int i = 1; i <= P; ++i) {
         T acc = hc[i];
 #pragma unroll
-        for (int i2 = i + 1; i2 <= P; ++i2) acc = fmad<T>(hc[i2], B[G::level_off(i2 - i) + sw.code[i][i2]], acc);
+        for (int i2 = i + 1; i2 <= P; ++i2)
+            acc = fmad<T>(hc[i2], B[RP::pos((int)G::level_off(i2 - i) + sw.code[i][i2])], acc);
         static_for<1, R + 1>([&](auto rc) {
             constexpr int r = decltype(rc)::value;
             constexpr int width = ipow(D, r);
             constexpr int off = trie_size(D, r - 1);
-            const T *run = B + G::level_off(P - i + r) + (int64_t)sw.code[i][P] * width;
+            const T *run = RP::kOn ? B + RP::pos((int)G::level_off(P - i + r) + sw.code[i][P] * width)
+                                   : B + G::level_off(P - i + r) + (int64_t)sw.code[i][P] * width;
 #pragma unroll
-            for (int iv = 0; iv < width; ++iv) acc = fmad<T>(hsub[off + iv], run[iv], acc);
+            for (int iv = 0; iv < width; ++iv) acc = fmad<T>(hsub[off + iv], run[RP::in_run(iv)], acc);
         });
         hc[i] = acc;
     }
@@ -716,7 +788,8 @@ __device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], 
             for (int iv = 0; iv < width; ++iv) {
                 T acc = hsub[off + iv];
 #pragma unroll
-                for (int e = 0; e < ext; ++e) acc = fmad<T>(hsub[offq + iv * ext + e], B[G::level_off(q) + e], acc);
+                for (int e = 0; e < ext; ++e)
+                    acc = fmad<T>(hsub[offq + iv * ext + e], B[RP::pos((int)G::level_off(q) + e)], acc);
                 hsub[off + iv] = acc;
             }
         });
@@ -731,7 +804,8 @@ __device__ __forceinline__ void contract_right(T (&hc)[P + 1], T (&hsub)[HSUB], 
 template <int D, int N, int P, int GW, typename T>
 constexpr size_t forward_lds_bytes() {
     using G = Geometry<D, N, P, sizeof(T)>;
-    return (size_t)GW * kTile * (N - P) * D * sizeof(T) + (size_t)(GW / 2) * G::kSigSize * sizeof(T);
+    return (size_t)GW * kTile * (N - P) * D * sizeof(T) +
+           (size_t)(GW / 2) * RowPlace<D, true>::size((int)G::kSigSize) * sizeof(T);
 }
 
 // LDS layout of the forward sweep: staged increments per chunk, and slots for the in-block products
@@ -740,7 +814,7 @@ struct ForwardShape {
     using G = Geometry<D, N, P, sizeof(T)>;
     static constexpr int KS = N - P;
     static constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
-    static constexpr int kSlotSize = GW > 1 ? (int)G::kSigSize : 4;
+    static constexpr int kSlotSize = GW > 1 ? RowPlace<D, true>::size((int)G::kSigSize) : 4;  // skewed rows
     static constexpr int kStage = kTile * KS * D;  // staged increments of one chunk
 };
 
@@ -861,9 +935,9 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             const bool right = (part % (2 * stride)) == stride;
             const bool left = (part % (2 * stride)) == 0;
             lds_barrier();
-            if (right && active) store_state<T, D, P, N, G::kFwdSub>(slot[pair], pu, a, sub);
+            if (right && active) store_state<T, D, P, N, G::kFwdSub, D, true>(slot[pair], pu, a, sub);
             lds_barrier();
-            if (left) apply_right<T, D, P, N, G::kFwdSub>(a, sub, slot[pair], sw);
+            if (left) apply_right<T, D, P, N, G::kFwdSub, true>(a, sub, slot[pair], sw);
         }
         if (part == 0 && active) store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
     } else {
@@ -1062,10 +1136,13 @@ constexpr int kCopyThreads = 128;
 
 // Copies one dense-layout row of COUNT elements with THREADS threads, in 16-byte pieces where the row
 // size allows; all loads of a thread are issued before its first store.
-template <typename T, int COUNT, int THREADS>
+// SKEW_D > 0: dst is a row in LDS in the layout of RowPlace<SKEW_D, true> (a piece never straddles its padding:
+// the pieces are at most four elements, and the layout moves whole groups of four).
+template <typename T, int COUNT, int THREADS, int SKEW_D = 0>
 __device__ __forceinline__ void copy_row(const T *src, T *dst, int tid) {
     using Stager = RowStager<T, COUNT, THREADS>;
     using V = typename Stager::V;
+    using RP = RowPlace<(SKEW_D > 0 ? SKEW_D : 4), (SKEW_D > 0)>;
     const V *s = reinterpret_cast<const V *>(src);
     V *d = reinterpret_cast<V *>(dst);
     V regs[Stager::kPer];
@@ -1077,7 +1154,7 @@ __device__ __forceinline__ void copy_row(const T *src, T *dst, int tid) {
 #pragma unroll
     for (int i = 0; i < Stager::kPer; ++i) {
         const int idx = i * THREADS + tid;
-        if (idx < Stager::kVecs) d[idx] = regs[i];
+        if (idx < Stager::kVecs) d[RP::kOn ? RP::pos(idx * Stager::kVW) / Stager::kVW : idx] = regs[i];
     }
 }
 
@@ -1498,11 +1575,12 @@ __device__ __forceinline__ void dense_backward_body(
         const SubWords<D, P> sw(u);
         // The lanes read the row of suffix products at addresses of their own, each entry several times over
         // the block: where the slab has room for it the row goes there first, in one coalesced copy.
-        constexpr bool kStageEdge = BS::kSlab && RowStager<T, (int)G::kLowSize, G::kBlock>::kPadded <= BS::kSlabElems;
+        // (in the skewed layout of rows in LDS, see RowPlace)
+        constexpr bool kStageEdge = BS::kSlab && RowPlace<D, true>::size((int)G::kLowSize) <= BS::kSlabElems;
         if constexpr (kStageEdge) {
-            copy_row<T, (int)G::kLowSize, G::kBlock>(edgeZ + unit * G::kLowSize, &slab[0], tid);
+            copy_row<T, (int)G::kLowSize, G::kBlock, D>(edgeZ + unit * G::kLowSize, &slab[0], tid);
             lds_barrier();
-            contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, &slab[0], sw);
+            contract_right<T, D, N, P, G::kFwdSub, true>(hc, hsub, &slab[0], sw);
         } else {
             contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
         }
