@@ -525,7 +525,7 @@ __device__ __forceinline__ void read_first_level(const T *sdx, int tt, int a0, T
 
 constexpr int pow2_divisor(int d) { return (d % 2 == 0) ? 2 * pow2_divisor(d / 2) : 1; }
 
-template <int D, int N, int P, int ELEM = 4>
+template <int D, int N, int P, int ELEM = 4, int MAXW = 0>
 struct Geometry {
     // A lane holds kK children of its prefix: all D, or fewer where the first level below the prefix is split
     // between kParts lanes (split_children).  The lanes of a part are padded to whole rows of sixteen lanes (the unit
@@ -554,8 +554,11 @@ struct Geometry {
     // fits: the reverse sweeps of these shapes spilled 200 to 400 registers to memory in blocks of eight or
     // sixteen waves.  Units of one block keep their shape (they may be cut into time chunks).
     static constexpr bool kSplit64 = ELEM == 8 && (kUnitWaves > kMaxWaves32 || (N - P >= 3 && kUnitWaves > 8));
+    // MAXW > 0: blocks of at most MAXW waves whatever the sub-trie (the sweeps with letter bounds run one wave to
+    // a block: see kLetterBlocks)
     static constexpr int kMaxWaves =
-        !kSplit64 ? kMaxWaves32
+        MAXW > 0 ? MAXW
+        : !kSplit64 ? kMaxWaves32
         : (kSubTrie >= 72 || N - P >= 3 || (kSubTrie >= 56 && P >= 6)) ? 4
         : kSubTrie >= 30 ? (kMaxWaves32 < 8 ? kMaxWaves32 : 8) : kMaxWaves32;
     // a unit of several blocks deals its waves out evenly (18 waves: three blocks of six, not 8 + 8 + 2 with six
@@ -568,6 +571,12 @@ struct Geometry {
     // swept in one piece, never cut into time chunks: units of several blocks, and units with split children (the
     // products of chunk signatures are not written for them)
     static constexpr bool kOnePiece = kUnitBlocks > 1 || kSplit;
+    // Sweeps with letter bounds: the waves of a unit differ in the words they leave out, by a factor of ten and
+    // more between the first letter 0 and the last, and a wave cannot issue faster than every fourth clock, so
+    // inside one block the unit takes as long as its longest wave takes alone.  With MAXW = 1 every wave is a block
+    // of its own (the unit's lanes never talk to each other inside a sweep; their per-increment sums meet in
+    // memory), the blocks of the longest waves are launched first, and the short ones fill in behind them.
+    static constexpr bool kLetterBlocks = MAXW > 0;
     static __host__ __device__ constexpr int64_t level_off(int k) {  // first column of level k in the dense layout
         int64_t o = 0, w = 1;
         for (int i = 1; i < k; ++i) {
@@ -588,6 +597,20 @@ __device__ __forceinline__ void prefix_letters(int pu, int (&u)[P]) {
         u[j] = pu % D;
         pu /= D;
     }
+}
+
+// Unit of the block, and which of the unit's blocks it is.  The blocks of a unit follow each other in the grid,
+// except in a launch of letter blocks: there all first blocks come first, then all second ones, .. (the blocks
+// with the smallest first letters, which leave out the fewest words, start first).
+template <typename G>
+__device__ __forceinline__ int64_t unit_of_block() {
+    if constexpr (G::kLetterBlocks) return (int64_t)(blockIdx.x % (gridDim.x / (unsigned)G::kUnitBlocks));
+    else return G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
+}
+template <typename G>
+__device__ __forceinline__ int part_of_block() {
+    if constexpr (G::kLetterBlocks) return (int)(blockIdx.x / (gridDim.x / (unsigned)G::kUnitBlocks));
+    else return (int)(blockIdx.x % (unsigned)G::kUnitBlocks);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -809,9 +832,9 @@ constexpr size_t forward_lds_bytes() {
 }
 
 // LDS layout of the forward sweep: staged increments per chunk, and slots for the in-block products
-template <typename T, int D, int N, int P, int GW>
+template <typename T, int D, int N, int P, int GW, int MAXW = 0>
 struct ForwardShape {
-    using G = Geometry<D, N, P, sizeof(T)>;
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
     static constexpr int KS = N - P;
     static constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
     static constexpr int kSlotSize = GW > 1 ? RowPlace<D, true>::size((int)G::kSigSize) : 4;  // skewed rows
@@ -823,16 +846,16 @@ struct ForwardShape {
 // chunk_low (optional): [rows, chunks, levels below N] receives every chunk's own signature below the top level.
 // BOUND: top-level words with a letter below BOUND after the prefix's first letter are left out (they stay zero
 // in the output); the LDS arrays belong to the calling kernel.
-template <typename T, int D, int N, int P, int GW, int BOUND>
+template <typename T, int D, int N, int P, int GW, int BOUND, int MAXW = 0>
 __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T *__restrict__ out,
                                                    const SigShape &shape, int chunks, T *__restrict__ zero_rows,
                                                    T *__restrict__ chunk_low,
                                                    const int pu,   // prefix of the thread within its chunk
                                                    const int tid,  // index of the thread within its chunk's block part
-                                                   T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW>::kStage],
-                                                   T (&slot)[ForwardShape<T, D, N, P, GW>::kSlots]
-                                                            [ForwardShape<T, D, N, P, GW>::kSlotSize]) {
-    using G = Geometry<D, N, P, sizeof(T)>;
+                                                   T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW, MAXW>::kStage],
+                                                   T (&slot)[ForwardShape<T, D, N, P, GW, MAXW>::kSlots]
+                                                            [ForwardShape<T, D, N, P, GW, MAXW>::kSlotSize]) {
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
     constexpr int KS = N - P;
     const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
     T *sdx = sdx_all[part];
@@ -847,7 +870,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
     prefix_letters<D, P>(active ? pp : 0, u);
 
     const int groups = chunks / GW;  // blocks per row
-    const int64_t blk = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
+    const int64_t blk = unit_of_block<G>();
     int64_t row, group_of_row, b, w;
     divide_index(blk, groups, row, group_of_row);
     const int c = (int)group_of_row * GW + part;
@@ -948,28 +971,30 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
 // BOUNDED: `bounds` holds the letter bounds of the wanted top-level words (see LetterBounds).  Every wave runs
 // the copy of the sweep compiled for its bound; the copies differ in nothing but the sub-trie nodes they leave
 // out, so all waves of the block still meet at the same barriers.
-template <typename T, int D, int N, int P, int GW, bool BOUNDED = false>
-__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock * GW))
+template <typename T, int D, int N, int P, int GW, bool BOUNDED = false, int MAXW = 0>
+__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
                          T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr,
                          T *__restrict__ chunk_low = nullptr) {
-    using FS = ForwardShape<T, D, N, P, GW>;
+    using FS = ForwardShape<T, D, N, P, GW, MAXW>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
     __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
-    using G = Geometry<D, N, P, sizeof(T)>;
-    static_assert(!G::kOnePiece || (GW == 1 && !BOUNDED), "a unit of several blocks is swept one chunk to a block");
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
+    static_assert(!G::kOnePiece || (GW == 1 && BOUNDED == G::kLetterBlocks),
+                  "a unit of several blocks is swept one chunk to a block; with letter bounds, in letter blocks");
     const int tid = (int)threadIdx.x % G::kBlock;
     if constexpr (BOUNDED) {
-        const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
+        const int pu = G::kLetterBlocks ? tid + part_of_block<G>() * G::kBlock : LetterBounds<D, P>::prefix_of_thread(tid);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
-            dense_forward_body<T, D, N, P, GW, decltype(loc)::value>(path, out, shape, chunks, zero_rows, chunk_low, pu,
-                                                                     tid, sdx_all, slot);
+            dense_forward_body<T, D, N, P, GW, decltype(loc)::value, MAXW>(path, out, shape, chunks, zero_rows,
+                                                                           chunk_low, pu, tid, sdx_all, slot);
         });
     } else {
-        const int pu = G::kUnitBlocks > 1 ? tid + (int)(blockIdx.x % G::kUnitBlocks) * G::kBlock : tid;
-        dense_forward_body<T, D, N, P, GW, 0>(path, out, shape, chunks, zero_rows, chunk_low, pu, tid, sdx_all, slot);
+        const int pu = G::kUnitBlocks > 1 ? tid + part_of_block<G>() * G::kBlock : tid;
+        dense_forward_body<T, D, N, P, GW, 0, MAXW>(path, out, shape, chunks, zero_rows, chunk_low, pu, tid, sdx_all,
+                                                    slot);
     }
 }
 
@@ -1018,6 +1043,17 @@ struct RowStager {
         for (int i = 0; i < kPer; ++i) {
             const int idx = i * BLOCK + (int)threadIdx.x;
             if (idx < kVecs) v[idx] = regs[i];
+        }
+    }
+    // into a row in the skewed layout of RowPlace<D, true>
+    template <int D>
+    __device__ __forceinline__ void commit_skewed(T *dst) const {
+        using RP = RowPlace<D, true>;
+        V *v = reinterpret_cast<V *>(dst);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int idx = i * BLOCK + (int)threadIdx.x;
+            if (idx < kVecs) v[RP::pos(idx * kVW) / kVW] = regs[i];
         }
     }
 };
@@ -1107,13 +1143,11 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
 // ---------------------------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------------------------
-// Adjoint state of a lane at the right end of a row: the upstream gradient.  Chain entries are
-// lane-private partial sums, so only the lane whose remaining prefix letters are zero starts from it.
-template <typename T, int D, int N, int P>
-__device__ __forceinline__ void load_adjoint(const T *__restrict__ grow, int pu, bool active, T (&hc)[P + 1],
-                                             T (&hsub)[Geometry<D, N, P>::kFwdSub], int a0 = 0) {
-    using G = Geometry<D, N, P>;
-    load_state<T, D, P, N, G::kFwdSub, G::kK>(grow, pu, active, hc, hsub, a0);
+// Adjoint state of a lane at the right end of a row: the upstream gradient (read like a signature state with
+// load_state).  Chain entries are lane-private partial sums, so only the lane whose remaining prefix letters are
+// zero keeps what it read.
+template <typename T, int D, int P>
+__device__ __forceinline__ void adjoint_chain_of_lane(int pu, int a0, T (&hc)[P + 1]) {
     int rest = 1;
 #pragma unroll
     for (int j = P; j >= 1; --j) {
@@ -1438,9 +1472,9 @@ __global__ void __launch_bounds__(kWave) chunk_level1_kernel(const T *__restrict
 // padded to kDP, into a slab of its wave (one or more 16-byte LDS stores), and once kSubTile increments have
 // gathered there the lanes read the slab back across the lanes, eight 16-byte reads each, and leave eight
 // partial sums per increment and letter in `sg`.
-template <typename T, int D, int N, int P>
+template <typename T, int D, int N, int P, int MAXW = 0>
 struct BackwardShape {
-    using G = Geometry<D, N, P, sizeof(T)>;
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
     static constexpr int KS = N - P;
     static constexpr int kDP = D <= 4 ? 4 : D <= 8 ? 8 : 16;  // letters padded to whole 16-byte pieces
     // (blocks of eight waves, their 64 KB of slabs in dynamic LDS and sums tiled by sixteen increments, measured
@@ -1453,8 +1487,10 @@ struct BackwardShape {
     static constexpr int kLetters = kSlab ? kDP : D;  // cells of one increment in a row of `sg`
     // LDS bytes of the parts of one increment
     static constexpr int kRowBytes = G::kWaves * kParts * kLetters * (int)sizeof(T);
+    // (letter blocks: eight one-wave blocks and their 8 KB slabs share a CU, so the sums of a tile take 4 KB)
+    static constexpr int kTileBytes = G::kLetterBlocks ? 4096 : 8192;
     static constexpr int kBwdTile =
-        kSlab ? (kRowBytes * 32 <= 8192 ? 32 : kRowBytes * 16 <= 8192 ? 16 : 8)
+        kSlab ? (kRowBytes * 32 <= kTileBytes ? 32 : kRowBytes * 16 <= kTileBytes ? 16 : 8)
               : (kRowBytes * 64 <= 49152 ? 64 : kRowBytes * 32 <= 49152 ? 32
                  : kRowBytes * 16 <= 131072 ? 16 : kRowBytes * 8 <= 131072 ? 8 : 4);
     // Increments are staged for several tiles at a time where that takes little LDS (at most 4 KB, plus the
@@ -1477,17 +1513,17 @@ struct BackwardShape {
 
 // BOUND: the upstream gradient is zero on every top-level word that has a letter below BOUND after the
 // prefix's first letter, and the sweep leaves those words out; the LDS arrays belong to the calling kernel.
-template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, int BOUND>
+template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, int BOUND, int MAXW = 0>
 __device__ __forceinline__ void dense_backward_body(
     const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig, const T *__restrict__ edgeA,
     const T *__restrict__ edgeZ, T *__restrict__ grad_inc, const SigShape &shape, int chunks, T *__restrict__ grad_path,
     const int pu_unit,  // index of the thread within its unit (its prefix, unless the first level is split)
     const int tid,      // index of the thread within its block
-    T (&sdx_all)[BackwardShape<T, D, N, P>::kStage],
-    T (&sg)[BackwardShape<T, D, N, P>::kSums][BackwardShape<T, D, N, P>::kSumRow],
-    T (&cells)[BackwardShape<T, D, N, P>::kCells], T (&slab)[BackwardShape<T, D, N, P>::kSlabElems], T (&carry)[D]) {
-    using G = Geometry<D, N, P, sizeof(T)>;
-    using BS = BackwardShape<T, D, N, P>;
+    T (&sdx_all)[BackwardShape<T, D, N, P, MAXW>::kStage],
+    T (&sg)[BackwardShape<T, D, N, P, MAXW>::kSums][BackwardShape<T, D, N, P, MAXW>::kSumRow],
+    T (&cells)[BackwardShape<T, D, N, P, MAXW>::kCells], T (&slab)[BackwardShape<T, D, N, P, MAXW>::kSlabElems], T (&carry)[D]) {
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
+    using BS = BackwardShape<T, D, N, P, MAXW>;
     constexpr int KS = N - P;
     constexpr int kParts = BS::kParts;
     constexpr int kBwdTile = BS::kBwdTile;
@@ -1511,7 +1547,7 @@ __device__ __forceinline__ void dense_backward_body(
         for (int k = 0; k < D; ++k) my_cells[k * G::kBlock] = T(0);
     }
 
-    int64_t unit = G::kUnitBlocks > 1 ? (int64_t)blockIdx.x / G::kUnitBlocks : (int64_t)blockIdx.x;
+    int64_t unit = unit_of_block<G>();
     if constexpr (CHUNKED && G::kUnitBlocks == 1) {
         // Consecutive blocks go to the eight XCDs in turn, each with an L2 of its own.  The chunks of a row read the
         // same upstream gradient, so they are dealt to one XCD: block b = 8 q + x works on the q-th unit of the
@@ -1560,32 +1596,40 @@ __device__ __forceinline__ void dense_backward_body(
             stage_increments<T, D, KS, G::kBlock>(sdx_all, x + staged_from * D, (int)(until - staged_from), tid);
         }
     };
-    if (ntiles > 0) stage_for(ntiles - 1);
-
     // A: signature at the right edge of the unit (levels < N).  H: adjoint at the right edge.
+    // Everything the prologue reads from memory is requested before the first wait: the upstream gradient, the two
+    // rows of chunk products, and last the path points of the first stage, whose wait is then the only one.
     constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
     T a[P + 1], hc[P + 1];
     T asub[kAS];
     T hsub[G::kFwdSub];
-    load_adjoint<T, D, N, P>(grow, pu, active, hc, hsub, a0);
+    load_state<T, D, P, N, G::kFwdSub, G::kK>(grow, pu, active, hc, hsub, a0);
     if constexpr (CHUNKED) {
         load_state<T, D, P, N - 1, kAS>(edgeA + unit * G::kLowSize, pu, active, a, asub);
         // adjoint at the right edge of the chunk: the upstream gradient contracted with the signature of
         // everything to the right of the chunk
         const SubWords<D, P> sw(u);
         // The lanes read the row of suffix products at addresses of their own, each entry several times over
-        // the block: where the slab has room for it the row goes there first, in one coalesced copy.
-        // (in the skewed layout of rows in LDS, see RowPlace)
+        // the block: where the slab has room for it the row goes there first, in one coalesced copy
+        // (in the skewed layout of rows in LDS, see RowPlace).
         constexpr bool kStageEdge = BS::kSlab && RowPlace<D, true>::size((int)G::kLowSize) <= BS::kSlabElems;
         if constexpr (kStageEdge) {
-            copy_row<T, (int)G::kLowSize, G::kBlock, D>(edgeZ + unit * G::kLowSize, &slab[0], tid);
+            RowStager<T, (int)G::kLowSize, G::kBlock> suffix_row;
+            suffix_row.fetch(edgeZ + unit * G::kLowSize);
+            if (ntiles > 0) stage_for(ntiles - 1);
+            suffix_row.template commit_skewed<D>(&slab[0]);
+            adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
             lds_barrier();
             contract_right<T, D, N, P, G::kFwdSub, true>(hc, hsub, &slab[0], sw);
         } else {
+            if (ntiles > 0) stage_for(ntiles - 1);
+            adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
             contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
         }
     } else {
         load_state<T, D, P, N - 1, kAS, KF>(sig + row * G::kSigSize, pu, active, a, asub, a0);
+        if (ntiles > 0) stage_for(ntiles - 1);
+        adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
     }
     a[0] = T(1);
     // onehot[j][k] = 1 when the j-th letter of the lane's prefix is k (kept in registers only where
@@ -1878,34 +1922,37 @@ __device__ __forceinline__ void dense_backward_body(
 // BOUNDED: the upstream gradient is zero on every top-level word outside the letter bounds in `bounds` (see
 // LetterBounds).  Every wave runs the copy of the sweep compiled for its bound; all copies meet at the same
 // barriers.
-template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, bool BOUNDED = false>
-__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T)>::kBlock))
+template <typename T, int D, int N, int P, bool ACCUMULATE, bool CHUNKED, bool BOUNDED = false, int MAXW = 0>
+__global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
                           const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
                           SigShape shape, int chunks, T *__restrict__ grad_path = nullptr,
                           const int *__restrict__ bounds = nullptr) {
-    using BS = BackwardShape<T, D, N, P>;
+    using BS = BackwardShape<T, D, N, P, MAXW>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx[BS::kStage];
     __shared__ __align__(16) T sg[BS::kSums][BS::kSumRow];
     __shared__ T cells[BS::kCells];
     __shared__ __align__(16) T slab[BS::kSlabElems];
     __shared__ T carry[D];  // kToPath: per-letter sums of the first increment of the tile flushed before
-    using G = Geometry<D, N, P, sizeof(T)>;
-    static_assert((G::kUnitBlocks == 1 || ACCUMULATE) && (!G::kOnePiece || (!CHUNKED && !BOUNDED)),
-                  "a unit of several blocks is swept in one piece and adds its per-increment sums in memory");
+    using G = Geometry<D, N, P, sizeof(T), MAXW>;
+    static_assert((G::kUnitBlocks == 1 || ACCUMULATE) &&
+                      (!G::kOnePiece || (G::kLetterBlocks ? (CHUNKED && BOUNDED) : (!CHUNKED && !BOUNDED))),
+                  "a unit of several blocks adds its per-increment sums in memory; it is swept in one piece, or, "
+                  "with letter bounds, in time chunks by letter blocks");
     const int tid = (int)threadIdx.x;
     if constexpr (BOUNDED) {
-        const int pu = LetterBounds<D, P>::prefix_of_thread(tid);
+        const int pu = G::kLetterBlocks ? tid + part_of_block<G>() * G::kBlock : LetterBounds<D, P>::prefix_of_thread(tid);
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
-            dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value>(
+            dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value, MAXW>(
                 path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry);
         });
     } else {
-        const int pu = G::kUnitBlocks > 1 ? tid + (int)(blockIdx.x % G::kUnitBlocks) * G::kBlock : tid;
-        dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0>(path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape,
-                                                                chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry);
+        const int pu = G::kUnitBlocks > 1 ? tid + part_of_block<G>() * G::kBlock : tid;
+        dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0, MAXW>(path, sig, grad_sig, edgeA, edgeZ, grad_inc,
+                                                                      shape, chunks, grad_path, pu, tid, sdx, sg, cells,
+                                                                      slab, carry);
     }
 }
 
@@ -2079,11 +2126,10 @@ void profile_mark(bool begin, hipStream_t stream) {
     if (!begin) g_profile.valid = true;
 }
 
-// number of time chunks per row: enough waves to give every SIMD of the GPU about two, but chunks
-// of at least 16 increments
-int pick_chunks(int64_t rows, int block, int64_t L) {
+// number of time chunks per row: enough waves to give every SIMD of the GPU about two (want_waves = 2048), but
+// chunks of at least 16 increments
+int pick_chunks(int64_t rows, int block, int64_t L, int64_t want_waves) {
     const int64_t waves_per_row = block / kWave;
-    const int64_t want_waves = 2048;
     int64_t c = (want_waves + rows * waves_per_row - 1) / (rows * waves_per_row);
     const int64_t max_c = (L - 1) / 16;
     if (c > max_c) c = max_c;
@@ -2160,9 +2206,18 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     int groups = chunks;
     if constexpr (kBoundsOk) {
         if (bounds) {
-            // bounded sweeps exist one chunk to a block only
-            hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)(rows * chunks)),
-                               dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds, chunk_low);
+            // bounded sweeps exist one chunk to a block only; in fp32 they run in letter blocks, one wave to a
+            // block (in fp64 a wave alone takes more registers than two of them have together on a SIMD)
+            if constexpr (sizeof(T) == 4) {
+                using GL = Geometry<D, N, P, sizeof(T), 1>;
+                hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true, 1>),
+                                   dim3((unsigned)(rows * chunks * GL::kUnitBlocks)), dim3(GL::kBlock), 0, stream, path,
+                                   chunk_sig, shape, chunks, (T *)nullptr, bounds, chunk_low);
+            } else {
+                hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 1, true>), dim3((unsigned)(rows * chunks)),
+                                   dim3(G::kBlock), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr, bounds,
+                                   chunk_low);
+            }
             groups = -1;
         }
     }
@@ -2237,7 +2292,9 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && !G::kOnePiece;
     const int64_t rows = shape.B * shape.W;
     // per-increment sums are added in memory for overlapping windows and for units spread over several blocks
-    const bool accumulate = shape.windows != nullptr || G::kUnitBlocks > 1;
+    // (among them the letter blocks of a sweep with letter bounds)
+    const bool accumulate =
+        shape.windows != nullptr || G::kUnitBlocks > 1 || (bounds != nullptr && kBoundsOk && sizeof(T) == 4);
     *wrote_path = false;
     hipError_t e;
     // bounded sweeps exist for time-chunked calls only (every call that embeds a projection is chunked)
@@ -2300,14 +2357,21 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         bool launched = false;
         if constexpr (kBoundsOk) {
             if (bounds) {
-                if (accumulate)
+                if constexpr (sizeof(T) == 4) {
+                    // letter blocks (see Geometry::kLetterBlocks): the per-increment sums meet in memory
+                    using GL = Geometry<D, N, P, sizeof(T), 1>;
+                    hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true, true, 1>),
+                                       dim3((unsigned)(units * GL::kUnitBlocks)), dim3(GL::kBlock), 0, stream, path, sig,
+                                       grad_sig, dumpA, dumpH, grad_inc, shape, chunks, (T *)nullptr, bounds);
+                } else if (accumulate) {
                     hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true, true>), dim3((unsigned)units),
                                        dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA,
                                        dumpH, grad_inc, shape, chunks, (T *)nullptr, bounds);
-                else
+                } else {
                     hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true, true>), dim3((unsigned)units),
                                        dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA,
                                        dumpH, grad_inc, shape, chunks, grad_path, bounds);
+                }
                 launched = true;
             }
         }
@@ -2403,7 +2467,8 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
             dc.bounded = chunks_ok && v.bounds_ok && level_sizes[depth] > 0 && level_sizes[depth] < top_dense &&
                          options().letter_bounds != 0;
         }
-        int chunks = pick_chunks(rows, v.block, L);
+        // (letter blocks: twice the waves that fit the GPU at once, so that the short ones fill in behind the long)
+        int chunks = pick_chunks(rows, v.block, L, dc.bounded && elem == 4 ? 4096 : 2048);
         // deep fp32 shapes: the reverse sweep rebuilds A_t = A_{t+1} (x) exp(-dx_t) step by step, and over a span of
         // large increments that roll-back loses digits at depth 9 and more (d = 2, depth 12, five increments of
         // size 0.8: gradient off by 1.5e-5 in one piece, 1e-6 in two or more); four chunks at least
