@@ -856,6 +856,29 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, set_option, dty
         assert rel_err(got, plain) < TOL[dtype] and rel_err(grad, plain_grad) < TOL[dtype]
 
 
+@pytest.mark.parametrize("d,depth", [(8, 5), (8, 4)])
+@pytest.mark.parametrize("chunks", [2, 3, 5])
+def test_letter_bounds_in_one_wave_blocks(ps, set_option, d, depth, chunks):
+    """fp32 sweeps with letter bounds run one wave to a block (the blocks of a first letter together in the grid,
+    the per-increment sums of a unit's waves added in memory): Lyndon projection at forced chunk counts, chunks of
+    unequal length, with and without windows, against the checker and against the run without bounds."""
+    set_option("chunks", chunks)
+    B, L = 3, 16 * chunks + 7
+    proj = ps.projections.lyndon(depth=depth, path_dim=d)
+    sizes, codes = _plan(proj)
+    path = brownian_path(B, L, d, seed=95) * 1.2
+    for windows in (None, [(0, L), (3, L - 2), (L // 2, L // 2 + 1)]):
+        want = TO.compute_signature(path, depth, sizes, codes, windows)
+        G = randn(tuple(want.shape), seed=96)
+        got, grad = _run_sig(ps, path, depth, torch.float32, projection=proj, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[torch.float32]
+        assert rel_err(grad, TO.signature_vjp(path, G, depth, sizes, codes, windows)) < TOL[torch.float32]
+        set_option("letter_bounds", 0)
+        plain, plain_grad = _run_sig(ps, path, depth, torch.float32, projection=proj, windows=windows, G=G)
+        set_option("letter_bounds", 1)
+        assert rel_err(got, plain) < TOL[torch.float32] and rel_err(grad, plain_grad) < TOL[torch.float32]
+
+
 # ------------------------------------------------------------------------------------------------
 # hand-over of the time-chunk signatures from the forward to the backward of one call
 # ------------------------------------------------------------------------------------------------
