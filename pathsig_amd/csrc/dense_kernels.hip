@@ -970,7 +970,8 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
 
 // BOUNDED: `bounds` holds the letter bounds of the wanted top-level words (see LetterBounds).  Every wave runs
 // the copy of the sweep compiled for its bound; the copies differ in nothing but the sub-trie nodes they leave
-// out, so all waves of the block still meet at the same barriers.
+// out, so all waves of the block still meet at the same barriers.  MAXW = 1: letter blocks, one wave to a block
+// (Geometry::kLetterBlocks).
 template <typename T, int D, int N, int P, int GW, bool BOUNDED = false, int MAXW = 0>
 __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
@@ -1580,8 +1581,7 @@ __device__ __forceinline__ void dense_backward_body(
     const int64_t ntiles = (len + kBwdTile - 1) / kBwdTile;
     const bool ghost = kToPath && len > 0 && begin > 0;
     // Increments reach LDS a stage at a time: the tiles ti - ti % kStageTiles .. ti share one (the leftmost stage
-    // also holds the ghost step).  The loads of the first stage are the first ones the kernel issues, so the loads
-    // of the state and of the upstream gradient below stay in flight while its increments are written.
+    // also holds the ghost step).  The first stage is requested last of the prologue's loads (below).
     constexpr int kStageTiles = BS::kStageTiles;
     int64_t staged_from = 0;  // first increment in `sdx_all`
     auto stage_for = [&](int64_t ti) {
