@@ -1968,7 +1968,7 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock))
 // lane) is taken.
 #define PSIG_VARIANTS(X) \
     X(0, 4, 6, 3, 5, 4) X(1, 8, 4, 2, 3, 2) X(2, 6, 5, 3, 3, 3) X(3, 4, 4, 2, 3, 2) X(4, 3, 5, 3, 4, 3) \
-    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 3, 3) X(7, 8, 4, 3, 3, 2) X(8, 3, 6, 3, 5, 4) X(9, 4, 5, 3, 4, 3) \
+    X(5, 2, 8, 5, 7, 6) X(6, 8, 5, 3, 4, 3) X(7, 8, 4, 3, 3, 2) X(8, 3, 6, 3, 5, 4) X(9, 4, 5, 3, 4, 3) \
     X(10, 5, 4, 2, 3, 2) X(11, 5, 5, 3, 4, 3) X(12, 5, 6, 4, 4, 4) X(13, 6, 4, 2, 3, 2) X(14, 7, 4, 2, 3, 2) \
     X(15, 7, 5, 3, 3, 3) X(16, 2, 2, 1, 1, 1) X(17, 3, 2, 1, 1, 1) X(18, 4, 2, 1, 1, 1) X(19, 5, 2, 1, 1, 1) \
     X(20, 6, 2, 1, 1, 1) X(21, 7, 2, 1, 1, 1) X(22, 8, 2, 1, 1, 1) X(23, 2, 3, 2, 2, 1) X(24, 3, 3, 2, 2, 1) \
