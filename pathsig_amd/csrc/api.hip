@@ -37,7 +37,7 @@ int64_t env_int(const char *name, int64_t fallback) {
 
 // Plain integers behind relaxed atomics: a setter on one thread and a call on another see whole values.
 struct OptionCells {
-    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share, tiled, deep_fp64;
+    std::atomic<int64_t> chunks, letter_bounds, logsig_scatter, batch_tile, embed_share, tiled, deep_fp64, grouped;
     OptionCells()
         : chunks(env_int("PATHSIG_CHUNKS", 0)),
           letter_bounds(getenv("PATHSIG_NO_LETTER_BOUNDS") ? 0 : 1),
@@ -45,7 +45,8 @@ struct OptionCells {
           batch_tile(env_int("PATHSIG_BATCH_TILE", 0)),
           embed_share(env_int("PATHSIG_EMBED_SHARE", -1)),
           tiled(getenv("PATHSIG_NO_TILED") ? 0 : 1),
-          deep_fp64(getenv("PATHSIG_NO_DEEP_FP64") ? 0 : 1) {}
+          deep_fp64(getenv("PATHSIG_NO_DEEP_FP64") ? 0 : 1),
+          grouped(getenv("PATHSIG_NO_GROUPED") ? 0 : 1) {}
 };
 OptionCells &option_cells() {
     static OptionCells cells;  // the environment is read here, once
@@ -63,6 +64,7 @@ const Options &options() {
     snapshot.embed_share = c.embed_share.load(std::memory_order_relaxed);
     snapshot.tiled = c.tiled.load(std::memory_order_relaxed);
     snapshot.deep_fp64 = c.deep_fp64.load(std::memory_order_relaxed);
+    snapshot.grouped = c.grouped.load(std::memory_order_relaxed);
     return snapshot;
 }
 
@@ -569,6 +571,8 @@ int pathsig_set_option(const char *name, int64_t value) {
         option_cells().tiled.store(value, std::memory_order_relaxed);
     } else if (!strcmp(name, "deep_fp64") && (value == 0 || value == 1)) {
         option_cells().deep_fp64.store(value, std::memory_order_relaxed);
+    } else if (!strcmp(name, "grouped") && (value == 0 || value == 1)) {
+        option_cells().grouped.store(value, std::memory_order_relaxed);
     } else {
         set_error("unknown option or value out of range: %s = %lld", name, (long long)value);
         return PATHSIG_ERR_ARGUMENT;

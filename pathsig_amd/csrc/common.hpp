@@ -55,6 +55,8 @@ struct Options {
     int64_t tiled;           // 0: every call takes the per-word kernels, whatever its shape (default 1)
     int64_t deep_fp64;       // 1 (default): fp32 backward calls of depth 9 and more run their sweep in fp64 (see
                              // backward_in_fp64 in api.hip); 0: in fp32 like every other call
+    int64_t grouped;         // 1 (default): a keeping fp32 forward hands the chunk products over by groups of four
+                             // chunks where that is compiled (DenseChoice::grouped); 0: one scan over all chunks
 };
 const Options &options();
 

@@ -19,6 +19,8 @@ struct DenseChoice {
     size_t backward_workspace;  // bytes of scratch the backward needs beyond the increment accumulator
     size_t keep_bytes;          // bytes the forward can keep for the backward: the prefix and suffix products of the
                                 // chunk signatures below the top level, or (resweep) the dense signature (0: none)
+    bool grouped;               // the kept products are those within groups of four chunks plus those of whole groups
+                                // (four arrays: [rows, chunks, low] twice, then [rows, chunks / 4, low] twice)
 };
 
 DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, const int64_t *level_sizes, int64_t B,

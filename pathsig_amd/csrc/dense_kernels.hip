@@ -839,6 +839,14 @@ struct ForwardShape {
     static constexpr int kSlots = GW / 2 > 0 ? GW / 2 : 1;
     static constexpr int kSlotSize = GW > 1 ? RowPlace<D, true>::size((int)G::kSigSize) : 4;  // skewed rows
     static constexpr int kStage = kTile * KS * D;  // staged increments of one chunk
+    // Grouped hand-over (blocks of four chunks, fp32): the block also leaves the products of its chunks with the
+    // chunks to their left and to their right inside the block (below the top level), which takes one more row below
+    // the top level in LDS.
+    static constexpr int kLowRow = RowPlace<D, true>::size((int)G::kLowSize);
+    static constexpr bool kGrouped =
+        GW == 4 && sizeof(T) == 4 && MAXW == 0 && N >= 4 && N - 1 >= P && !G::kOnePiece &&
+        ((size_t)GW * kStage + (size_t)kSlots * kSlotSize + kLowRow) * sizeof(T) <= 64 * 1024;
+    static constexpr int kLowSlot = kGrouped ? kLowRow : 4;
 };
 
 // zero_rows (optional, GW = 1): the block also clears the points of its chunk in a [B, L, D] buffer (the last
@@ -854,8 +862,11 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
                                                    const int tid,  // index of the thread within its chunk's block part
                                                    T (&sdx_all)[GW][ForwardShape<T, D, N, P, GW, MAXW>::kStage],
                                                    T (&slot)[ForwardShape<T, D, N, P, GW, MAXW>::kSlots]
-                                                            [ForwardShape<T, D, N, P, GW, MAXW>::kSlotSize]) {
+                                                            [ForwardShape<T, D, N, P, GW, MAXW>::kSlotSize],
+                                                   T (&lowslot)[ForwardShape<T, D, N, P, GW, MAXW>::kLowSlot],
+                                                   T *__restrict__ group_suffix) {
     using G = Geometry<D, N, P, sizeof(T), MAXW>;
+    using FS = ForwardShape<T, D, N, P, GW, MAXW>;
     constexpr int KS = N - P;
     const int part = (int)threadIdx.x / G::kBlock;  // chunk within the block
     T *sdx = sdx_all[part];
@@ -945,6 +956,56 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             }
         }
     }
+    if constexpr (FS::kGrouped) {
+        if (group_suffix != nullptr) {
+            // Grouped hand-over.  The four chunks of the block are c0 .. c3; chunk_low receives, per chunk j, the
+            // product c0 (x) .. (x) cj, group_suffix the product c(j+1) (x) .. (x) c3 (nothing for j = 3: the
+            // identity), both below the top level; `out` receives the product of all four as before.  The products
+            // that the block's result does not need run on the waves that would otherwise wait:
+            //   round 1   wave 0: c0 (x) c1          wave 2: c2 (x) c3
+            //   round 2   wave 0: (c0 c1) (x) (c2 c3)   wave 1: c1 (x) (c2 c3)   wave 3: (c0 c1) (x) c2   (the last two
+            //             below the top level)
+            constexpr int kLow = (int)G::kLowSize;
+            const SubWords<D, P> sw(u);
+            T *prefix_at = chunk_low + (row * chunks + c) * kLow;
+            T *suffix_at = group_suffix + (row * chunks + c) * kLow;
+            if (part == 0 && active) store_state<T, D, P, N - 1, G::kFwdSub>(prefix_at, pu, a, sub);
+            if (part == 3 && active) store_state<T, D, P, N - 1, G::kFwdSub>(suffix_at - kLow, pu, a, sub);
+            if (part == 1 && active) store_state<T, D, P, N, G::kFwdSub, D, true>(slot[0], pu, a, sub);
+            if (part == 3 && active) store_state<T, D, P, N, G::kFwdSub, D, true>(slot[1], pu, a, sub);
+            if (part == 2 && active) store_state<T, D, P, N - 1, G::kFwdSub, D, true>(lowslot, pu, a, sub);
+            lds_barrier();
+            if (part == 0) apply_right<T, D, P, N, G::kFwdSub, true>(a, sub, slot[0], sw);
+            if (part == 2) apply_right<T, D, P, N, G::kFwdSub, true>(a, sub, slot[1], sw);
+            lds_barrier();
+            if (part == 0 && active) {
+                store_state<T, D, P, N - 1, G::kFwdSub>(prefix_at + kLow, pu, a, sub);
+                store_state<T, D, P, N - 1, G::kFwdSub, D, true>(slot[1], pu, a, sub);
+            }
+            if (part == 2 && active) {
+                store_state<T, D, P, N - 1, G::kFwdSub>(suffix_at - kLow, pu, a, sub);
+                store_state<T, D, P, N, G::kFwdSub, D, true>(slot[0], pu, a, sub);
+            }
+            lds_barrier();
+            if (part == 0) {
+                apply_right<T, D, P, N, G::kFwdSub, true>(a, sub, slot[0], sw);
+                if (active) {
+                    store_state<T, D, P, N - 1, G::kFwdSub>(prefix_at + 3 * kLow, pu, a, sub);
+                    store_state<T, D, P, N, G::kFwdSub>(out + blk * G::kSigSize, pu, a, sub);
+                }
+            }
+            if (part == 1) {
+                apply_right<T, D, P, N - 1, G::kFwdSub, true>(a, sub, slot[0], sw);
+                if (active) store_state<T, D, P, N - 1, G::kFwdSub>(suffix_at - kLow, pu, a, sub);
+            }
+            if (part == 3) {
+                load_state<T, D, P, N - 1, G::kFwdSub, D, true>(slot[1], pu, active, a, sub);
+                apply_right<T, D, P, N - 1, G::kFwdSub, true>(a, sub, lowslot, sw);
+                if (active) store_state<T, D, P, N - 1, G::kFwdSub>(prefix_at - kLow, pu, a, sub);
+            }
+            return;
+        }
+    }
     if constexpr (N - 1 >= P) {
         // the chunk's own signature below the top level, kept for the backward of the same call
         if (chunk_low != nullptr && active)
@@ -976,11 +1037,12 @@ template <typename T, int D, int N, int P, int GW, bool BOUNDED = false, int MAX
 __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock * GW))
     dense_forward_kernel(const T *__restrict__ path, T *__restrict__ out, SigShape shape, int chunks,
                          T *__restrict__ zero_rows = nullptr, const int *__restrict__ bounds = nullptr,
-                         T *__restrict__ chunk_low = nullptr) {
+                         T *__restrict__ chunk_low = nullptr, T *__restrict__ group_suffix = nullptr) {
     using FS = ForwardShape<T, D, N, P, GW, MAXW>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx_all[GW][FS::kStage];
     __shared__ __align__(16) T slot[FS::kSlots][FS::kSlotSize];
+    __shared__ __align__(16) T lowslot[FS::kLowSlot];
     using G = Geometry<D, N, P, sizeof(T), MAXW>;
     static_assert(!G::kOnePiece || (GW == 1 && BOUNDED == G::kLetterBlocks),
                   "a unit of several blocks is swept one chunk to a block; with letter bounds, in letter blocks");
@@ -990,12 +1052,13 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock * 
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_forward_body<T, D, N, P, GW, decltype(loc)::value, MAXW>(path, out, shape, chunks, zero_rows,
-                                                                           chunk_low, pu, tid, sdx_all, slot);
+                                                                           chunk_low, pu, tid, sdx_all, slot, lowslot,
+                                                                           (T *)nullptr);
         });
     } else {
         const int pu = G::kUnitBlocks > 1 ? tid + part_of_block<G>() * G::kBlock : tid;
         dense_forward_body<T, D, N, P, GW, 0, MAXW>(path, out, shape, chunks, zero_rows, chunk_low, pu, tid, sdx_all,
-                                                    slot);
+                                                    slot, lowslot, group_suffix);
     }
 }
 
@@ -1073,9 +1136,12 @@ struct CombineShape {
 
 // (the first BLOCK threads of the block, on the lanes lane_base .. lane_base + BLOCK - 1 of the row; sB: two buffers
 // of CombineShape::kStage elements)
+// running_low (optional): [rows, chunks, levels below N] receives, at chunk c >= 1, the product of the chunks before
+// c below the top level.
 template <typename T, int D, int N, int P, int BLOCK = Geometry<D, N, P>::kBlock>
 __device__ __forceinline__ void combine_staged(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks,
-                                               int64_t row, T *sB0, T *sB1, int lane_base = 0) {
+                                               int64_t row, T *sB0, T *sB1, int lane_base = 0,
+                                               T *__restrict__ running_low = nullptr) {
     using G = Geometry<D, N, P>;
     constexpr int kAhead = 3;
     const int pu = lane_base + (int)threadIdx.x;
@@ -1104,6 +1170,10 @@ __device__ __forceinline__ void combine_staged(const T *__restrict__ chunk_sig, 
             constexpr int qn = (q + 1) % kAhead;  // register set of the next chunk
             const int c = base + q;
             if (c < chunks) {
+                if constexpr (N - 1 >= P) {
+                    if (running_low != nullptr && active)
+                        store_state<T, D, P, N - 1, G::kFwdSub>(running_low + (row * chunks + c) * G::kLowSize, pu, a, sub);
+                }
                 apply_right<T, D, P, N, G::kFwdSub>(a, sub, (c & 1) ? sB1 : sB0, sw);
                 stager[qn].commit(((c + 1) & 1) ? sB1 : sB0);
                 const int nxt = c + 1 + kAhead;
@@ -1432,6 +1502,58 @@ __global__ void __launch_bounds__((EdgesShape<T, D, N, PS, PC>::kThreads))
     else scan_resident<T, D, N, PS, false>(chunk_low, edgeZ, chunks, resident, row, dyn, sOut[0], sOut[1]);
 }
 
+// Grouped hand-over: the products of whole groups of four chunks.  `partial` holds the `groups` group products of
+// every row (dense-layout rows, the forward sweep's block results).
+//   blockIdx.y == 0:  edgeR_g = Q_{g+1} (x) .. (x) Q_{groups-1} below the top level, g = 0 .. groups - 2
+//   blockIdx.y >= 1:  the signature of the row (combine_staged), which on its way leaves
+//                     edgeL_g = Q_0 (x) .. (x) Q_{g-1} below the top level, g = 1 .. groups - 1
+// (both arrays [rows, groups, levels below N]; the entries not named are never read)
+template <typename T, int D, int N, int PS, int PC>
+__global__ void __launch_bounds__((EdgesShape<T, D, N, PS, PC>::kThreads))
+    dense_group_edges_kernel(const T *__restrict__ partial, T *__restrict__ edgeL, T *__restrict__ edgeR,
+                             T *__restrict__ sig, int groups) {
+    using ES = EdgesShape<T, D, N, PS, PC>;
+    using G = Geometry<D, N, PS>;
+    extern __shared__ __align__(16) unsigned char group_smem[];
+    __shared__ __align__(16) T sOut[2][ES::kLow];
+    T *dyn = reinterpret_cast<T *>(group_smem);
+    const int64_t row = blockIdx.x;
+    if (blockIdx.y >= 1) {
+        if ((int)threadIdx.x >= ES::kCombineBlock) return;
+        combine_staged<T, D, N, PC, ES::kCombineBlock>(partial, sig, groups, row, dyn,
+                                                       dyn + CombineShape<T, D, N, PC, ES::kCombineBlock>::kStage,
+                                                       ((int)blockIdx.y - 1) * ES::kCombineBlock, edgeL);
+        return;
+    }
+    if ((int)threadIdx.x >= G::kBlock) return;
+    constexpr int kAS = G::kASub > 0 ? G::kASub : 1;
+    constexpr int kLow = ES::kLow;
+    const int pu = (int)threadIdx.x;
+    const bool active = (G::kLanes == G::kBlock) || pu < G::kLanes;
+    int u[PS];
+    prefix_letters<D, PS>(active ? pu : 0, u);
+    const SubWords<D, PS> sw(u);
+    const T *rows = partial + row * groups * G::kSigSize;
+    T *edge = edgeR + row * groups * kLow;
+    T a[PS + 1];
+    T asub[kAS];
+    // R_{groups-2} = Q_{groups-1}; R_{g-1} = Q_g (x) R_g
+    load_state<T, D, PS, N - 1, kAS>(rows + (int64_t)(groups - 1) * G::kSigSize, pu, active, a, asub);
+    if (active) {
+        store_state<T, D, PS, N - 1, kAS>(sOut[(groups - 2) & 1], pu, a, asub);
+        store_state<T, D, PS, N - 1, kAS>(edge + (int64_t)(groups - 2) * kLow, pu, a, asub);
+    }
+    for (int g = groups - 2; g >= 1; --g) {
+        load_state<T, D, PS, N - 1, kAS>(rows + (int64_t)g * G::kSigSize, pu, active, a, asub);
+        lds_barrier();
+        apply_right<T, D, PS, N - 1, kAS>(a, asub, sOut[g & 1], sw);
+        if (active) {
+            store_state<T, D, PS, N - 1, kAS>(sOut[(g - 1) & 1], pu, a, asub);
+            store_state<T, D, PS, N - 1, kAS>(edge + (int64_t)(g - 1) * kLow, pu, a, asub);
+        }
+    }
+}
+
 // Depth 2: the signature of a chunk below the top level is its level 1, the sum of its increments.  One block
 // per (row, chunk); zero_rows as in dense_forward_kernel (the block also clears the points of its chunk in a
 // [B, L, d] buffer, the last chunk of a row the final point too).
@@ -1522,7 +1644,8 @@ __device__ __forceinline__ void dense_backward_body(
     const int tid,      // index of the thread within its block
     T (&sdx_all)[BackwardShape<T, D, N, P, MAXW>::kStage],
     T (&sg)[BackwardShape<T, D, N, P, MAXW>::kSums][BackwardShape<T, D, N, P, MAXW>::kSumRow],
-    T (&cells)[BackwardShape<T, D, N, P, MAXW>::kCells], T (&slab)[BackwardShape<T, D, N, P, MAXW>::kSlabElems], T (&carry)[D]) {
+    T (&cells)[BackwardShape<T, D, N, P, MAXW>::kCells], T (&slab)[BackwardShape<T, D, N, P, MAXW>::kSlabElems], T (&carry)[D],
+    const T *__restrict__ edgeL = nullptr, const T *__restrict__ edgeR = nullptr) {
     using G = Geometry<D, N, P, sizeof(T), MAXW>;
     using BS = BackwardShape<T, D, N, P, MAXW>;
     constexpr int KS = N - P;
@@ -1605,7 +1728,7 @@ __device__ __forceinline__ void dense_backward_body(
     T hsub[G::kFwdSub];
     load_state<T, D, P, N, G::kFwdSub, G::kK>(grow, pu, active, hc, hsub, a0);
     if constexpr (CHUNKED) {
-        load_state<T, D, P, N - 1, kAS>(edgeA + unit * G::kLowSize, pu, active, a, asub);
+        auto load_edge_state = [&](const T *edge_row) { load_state<T, D, P, N - 1, kAS>(edge_row, pu, active, a, asub); };
         // adjoint at the right edge of the chunk: the upstream gradient contracted with the signature of
         // everything to the right of the chunk
         const SubWords<D, P> sw(u);
@@ -1613,7 +1736,61 @@ __device__ __forceinline__ void dense_backward_body(
         // the block: where the slab has room for it the row goes there first, in one coalesced copy
         // (in the skewed layout of rows in LDS, see RowPlace).
         constexpr bool kStageEdge = BS::kSlab && RowPlace<D, true>::size((int)G::kLowSize) <= BS::kSlabElems;
-        if constexpr (kStageEdge) {
+        if constexpr (kStageEdge && N >= 4 && N - 1 >= P && sizeof(T) == 4) {
+            if (edgeL != nullptr) {
+                // Grouped hand-over: edgeA / edgeZ hold the products of the chunk with the chunks to its left / to
+                // its right inside its group of four, edgeL / edgeR those of the groups to the left / right of the
+                // group (all below the top level).  A = L (x) A_in;  H = G contracted with Z_in (x) R.
+                const int grp = c >> 2, in_grp = c & 3, groups = chunks >> 2;
+                const bool have_right = grp < groups - 1, have_rest = in_grp < 3, have_left = grp > 0;
+                const int64_t group_row = (row * groups + grp) * G::kLowSize;
+                using Stager = RowStager<T, (int)G::kLowSize, G::kBlock>;
+                // (rows that are not needed are read all the same, from places that exist: loads under a
+                // condition would make the compiler wait for everything at their first use)
+                Stager right_row, own_row;
+                T z[P + 1], zsub[kAS];  // the product to the right inside the group, as a lane state
+                right_row.fetch(edgeR + (have_right ? group_row : (int64_t)0));
+                load_state<T, D, P, N - 1, kAS>(edgeZ + unit * G::kLowSize, pu, active, z, zsub);
+                own_row.fetch(edgeA + unit * G::kLowSize);
+                load_edge_state(have_left ? edgeL + group_row : edgeA + unit * G::kLowSize);
+                if (ntiles > 0) stage_for(ntiles - 1);
+                adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
+                // suffix of the rest of the row, Z = Z_in (x) R: a product below the top level on the lanes' states
+                // (a second contraction of the full adjoint would cost three times as much), handed to the
+                // contraction through the slab
+                if (have_right) {
+                    right_row.template commit_skewed<D>(&slab[0]);
+                    lds_barrier();
+                    if (have_rest) {
+                        apply_right<T, D, P, N - 1, kAS, true>(z, zsub, &slab[0], sw);
+                        lds_barrier();
+                    }
+                }
+                if (have_rest) {
+                    if (active) store_state<T, D, P, N - 1, kAS, D, true>(&slab[0], pu, z, zsub);
+                    lds_barrier();
+                }
+                if (have_right || have_rest) {
+                    contract_right<T, D, N, P, G::kFwdSub, true>(hc, hsub, &slab[0], sw);
+                    lds_barrier();
+                }
+                if (have_left) {
+                    own_row.template commit_skewed<D>(&slab[0]);
+                    lds_barrier();
+                    apply_right<T, D, P, N - 1, kAS, true>(a, asub, &slab[0], sw);
+                }
+            } else {
+                load_edge_state(edgeA + unit * G::kLowSize);
+                RowStager<T, (int)G::kLowSize, G::kBlock> suffix_row;
+                suffix_row.fetch(edgeZ + unit * G::kLowSize);
+                if (ntiles > 0) stage_for(ntiles - 1);
+                suffix_row.template commit_skewed<D>(&slab[0]);
+                adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
+                lds_barrier();
+                contract_right<T, D, N, P, G::kFwdSub, true>(hc, hsub, &slab[0], sw);
+            }
+        } else if constexpr (kStageEdge) {
+            load_edge_state(edgeA + unit * G::kLowSize);
             RowStager<T, (int)G::kLowSize, G::kBlock> suffix_row;
             suffix_row.fetch(edgeZ + unit * G::kLowSize);
             if (ntiles > 0) stage_for(ntiles - 1);
@@ -1622,6 +1799,7 @@ __device__ __forceinline__ void dense_backward_body(
             lds_barrier();
             contract_right<T, D, N, P, G::kFwdSub, true>(hc, hsub, &slab[0], sw);
         } else {
+            load_edge_state(edgeA + unit * G::kLowSize);
             if (ntiles > 0) stage_for(ntiles - 1);
             adjoint_chain_of_lane<T, D, P>(pu, a0, hc);
             contract_right<T, D, N, P, G::kFwdSub>(hc, hsub, edgeZ + unit * G::kLowSize, sw);
@@ -1927,7 +2105,8 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock))
     dense_backward_kernel(const T *__restrict__ path, const T *__restrict__ sig, const T *__restrict__ grad_sig,
                           const T *__restrict__ edgeA, const T *__restrict__ edgeZ, T *__restrict__ grad_inc,
                           SigShape shape, int chunks, T *__restrict__ grad_path = nullptr,
-                          const int *__restrict__ bounds = nullptr) {
+                          const int *__restrict__ bounds = nullptr, const T *__restrict__ edgeL = nullptr,
+                          const T *__restrict__ edgeR = nullptr) {
     using BS = BackwardShape<T, D, N, P, MAXW>;
     static_assert(!BOUNDED || LetterBounds<D, P>::kUsable, "letter bounds need one first letter per wave");
     __shared__ __align__(16) T sdx[BS::kStage];
@@ -1946,13 +2125,14 @@ __global__ void __launch_bounds__((Geometry<D, N, P, sizeof(T), MAXW>::kBlock))
         const int lo = LetterBounds<D, P>::of_wave(bounds, pu);
         dispatch_value<0, D>(lo, [&](auto loc) {
             dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, decltype(loc)::value, MAXW>(
-                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry);
+                path, sig, grad_sig, edgeA, edgeZ, grad_inc, shape, chunks, grad_path, pu, tid, sdx, sg, cells, slab, carry,
+                edgeL, edgeR);
         });
     } else {
         const int pu = G::kUnitBlocks > 1 ? tid + part_of_block<G>() * G::kBlock : tid;
         dense_backward_body<T, D, N, P, ACCUMULATE, CHUNKED, 0, MAXW>(path, sig, grad_sig, edgeA, edgeZ, grad_inc,
                                                                       shape, chunks, grad_path, pu, tid, sdx, sg, cells,
-                                                                      slab, carry);
+                                                                      slab, carry, edgeL, edgeR);
     }
 }
 
@@ -2054,9 +2234,28 @@ struct VariantInfo {
     bool bounds_ok;       // the sweeps can leave out top-level words by letter bounds
     bool chunks_ok[2];    // fp32, fp64: rows can be cut into time chunks
     bool fp64_fits;       // a lane's state fits the register file in fp64 too (else a later entry of the shape serves fp64)
+    bool grouped_ok;      // fp32: the hand-over of chunk products by groups of four chunks is compiled
 };
 
-template <int D, int N, int P, int PS>
+// Grouped hand-over (fp32): the forward sweep, four chunks to a block, leaves the products of every chunk with its
+// neighbours inside the block, a small launch the products of whole blocks, and the reverse sweep puts the two
+// together (one more contraction and one more product per chunk in its prologue).  It replaces the scan over all
+// chunks of a row, fifteen dependent products per direction and twice the chunk rows through memory.
+template <int D, int N, int P, int PC, int PS>
+constexpr bool grouped_handover_ok() {
+    if constexpr (N < 4 || N - 1 < P) {
+        return false;
+    } else {
+        using G = Geometry<D, N, P, 4>;
+        using BS = BackwardShape<float, D, N, P>;
+        constexpr bool staged = 2 * Geometry<D, N, PC>::kSigSize * sizeof(float) <= 48 * 1024;
+        return ForwardShape<float, D, N, P, 4>::kGrouped && G::kBlock * 4 <= 1024 && staged &&
+               EdgesShape<float, D, N, PS, PC>::kUsable && scan_fits<float, D, N, PS>() && BS::kSlab &&
+               RowPlace<D, true>::size((int)G::kLowSize) <= BS::kSlabElems;
+    }
+}
+
+template <int D, int N, int P, int PC, int PS>
 constexpr VariantInfo variant_info() {
     using G = Geometry<D, N, P>;
     using G64 = Geometry<D, N, P, 8>;
@@ -2064,7 +2263,8 @@ constexpr VariantInfo variant_info() {
                        LetterBounds<D, P>::kUsable && !G::kOnePiece && D <= 16,
                        {!G::kOnePiece && scan_fits<float, D, N, PS>(),
                         !G64::kOnePiece && scan_fits<double, D, N, PS>()},
-                       G::kSplit || trie_size(D, N - P) <= 132};
+                       G::kSplit || trie_size(D, N - P) <= 132,
+                       grouped_handover_ok<D, N, P, PC, PS>()};
 }
 
 constexpr size_t kBoundsBytes = 256;  // scratch for the letter bounds (16 ints, padded)
@@ -2098,13 +2298,13 @@ constexpr bool shape_enabled(int d, int depth) {
 constexpr bool shape_enabled(int, int) { return true; }
 #endif
 
-template <int D, int N, int P, int PS>
+template <int D, int N, int P, int PC, int PS>
 constexpr VariantInfo variant_info_if_enabled() {
-    if constexpr (shape_enabled(D, N)) return variant_info<D, N, P, PS>();
-    else return VariantInfo{-1, -1, 0, 0, 0, 0, false, {false, false}, false};
+    if constexpr (shape_enabled(D, N)) return variant_info<D, N, P, PC, PS>();
+    else return VariantInfo{-1, -1, 0, 0, 0, 0, false, {false, false}, false, false};
 }
 
-#define PSIG_INFO(I, D, N, P, PC, PS) variant_info_if_enabled<D, N, P, PS>(),
+#define PSIG_INFO(I, D, N, P, PC, PS) variant_info_if_enabled<D, N, P, PC, PS>(),
 constexpr VariantInfo kVariants[] = {PSIG_VARIANTS(PSIG_INFO)};
 #undef PSIG_INFO
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -2175,7 +2375,7 @@ hipError_t launch_scan(const T *chunk_low, T *edgeA, T *edgeZ, int64_t rows, int
 // pad256 bytes after the start of the first.
 template <typename T, int D, int N, int P, int PC, int PS>
 hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks, const int *bounds, T *keep,
-                       void *workspace, hipStream_t stream) {
+                       void *workspace, hipStream_t stream, bool grouped) {
     using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PC>;
     constexpr bool kStaged = 2 * GC::kSigSize * sizeof(T) <= 48 * 1024;
@@ -2203,6 +2403,33 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     // the chunks' own signatures below the top level, from which the products for the backward are made
     T *chunk_low = keep ? (T *)((unsigned char *)workspace + pad256((size_t)rows * chunks * G::kSigSize * sizeof(T)))
                         : (T *)nullptr;
+    if constexpr (sizeof(T) == 4 && grouped_handover_ok<D, N, P, PC, PS>()) {
+        if (keep && grouped && !bounds && chunks % 4 == 0 && chunks >= 8) {
+            // grouped hand-over: keep = [in-group prefix products][in-group suffix products], both
+            // [rows, chunks, low], then [products of the groups to the left][.. to the right], both
+            // [rows, chunks / 4, low]
+            using ES = EdgesShape<T, D, N, PS, PC>;
+            const int groups4 = chunks / 4;
+            const size_t unit_bytes = pad256((size_t)rows * chunks * G::kLowSize * sizeof(T));
+            const size_t group_bytes = pad256((size_t)rows * groups4 * G::kLowSize * sizeof(T));
+            T *in_suffix = (T *)((unsigned char *)keep + unit_bytes);
+            T *edgeL = (T *)((unsigned char *)keep + 2 * unit_bytes);
+            T *edgeR = (T *)((unsigned char *)keep + 2 * unit_bytes + group_bytes);
+            hipLaunchKernelGGL((dense_forward_kernel<T, D, N, P, 4>), dim3((unsigned)(rows * groups4)),
+                               dim3(G::kBlock * 4), 0, stream, path, chunk_sig, shape, chunks, (T *)nullptr,
+                               (const int *)nullptr, keep, in_suffix);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            auto kernel = dense_group_edges_kernel<T, D, N, PS, PC>;
+            if (ES::kCombineBytes > 48 * 1024) {
+                e = allow_dynamic_lds<dense_group_edges_kernel<T, D, N, PS, PC>>(ES::kCombineBytes);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)rows, 1 + ES::kCombineParts), dim3(ES::kThreads),
+                               ES::kCombineBytes, stream, (const T *)chunk_sig, edgeL, edgeR, sig, groups4);
+            return hipGetLastError();
+        }
+    }
     int groups = chunks;
     if constexpr (kBoundsOk) {
         if (bounds) {
@@ -2283,10 +2510,10 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
     }
 }
 
-template <typename T, int D, int N, int P, int PS>
+template <typename T, int D, int N, int P, int PC, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
                         const SigShape &shape, int chunks, const int *bounds, const T *kept, void *workspace,
-                        hipStream_t stream) {
+                        hipStream_t stream, bool grouped) {
     using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PS>;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && !G::kOnePiece;
@@ -2327,10 +2554,18 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
         const int64_t units = rows * chunks;
         const size_t edge_bytes = pad256((size_t)units * G::kLowSize * sizeof(T));
         const T *dumpA, *dumpH;
+        const T *edgeL = nullptr, *edgeR = nullptr;  // grouped hand-over: products of whole groups of chunks
         if (kept) {
             // the forward of this call left the prefix and suffix products of its chunk signatures
             dumpA = kept;
             dumpH = (const T *)((const unsigned char *)kept + edge_bytes);
+            if constexpr (sizeof(T) == 4 && grouped_handover_ok<D, N, P, PC, PS>()) {
+                if (grouped && !bounds && chunks % 4 == 0 && chunks >= 8) {
+                    const size_t group_bytes = pad256((size_t)rows * (chunks / 4) * G::kLowSize * sizeof(T));
+                    edgeL = (const T *)((const unsigned char *)kept + 2 * edge_bytes);
+                    edgeR = (const T *)((const unsigned char *)kept + 2 * edge_bytes + group_bytes);
+                }
+            }
         } else {
             unsigned char *ws = (unsigned char *)workspace;
             T *chunk_low = (T *)ws;
@@ -2379,11 +2614,11 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
             if (accumulate)
                 hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, true, true>), dim3((unsigned)units),
                                    dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA, dumpH,
-                                   grad_inc, shape, chunks, (T *)nullptr);
+                                   grad_inc, shape, chunks, (T *)nullptr, (const int *)nullptr, edgeL, edgeR);
             else
                 hipLaunchKernelGGL((dense_backward_kernel<T, D, N, P, false, true>), dim3((unsigned)units),
                                    dim3(G::kBlock), 0, stream, path, sig, grad_sig, dumpA, dumpH,
-                                   grad_inc, shape, chunks, grad_path);
+                                   grad_inc, shape, chunks, grad_path, (const int *)nullptr, edgeL, edgeR);
         }
         if (!accumulate) *wrote_path = true;
         profile_bracket(false, stream);
@@ -2491,8 +2726,13 @@ DenseChoice dense_choice(size_t elem, int64_t d, int depth, bool all_dense, cons
                                     pad256((size_t)rows * dc.fwd_chunks * v.low_size * elem);
         if (dc.bwd_chunks > 1) dc.backward_workspace += 3 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
         // the forward can hand those products to the backward when both cut the rows the same way
-        if (dc.bwd_chunks > 1 && dc.fwd_chunks == dc.bwd_chunks)
+        if (dc.bwd_chunks > 1 && dc.fwd_chunks == dc.bwd_chunks) {
             dc.keep_bytes = 2 * pad256((size_t)rows * dc.bwd_chunks * v.low_size * elem);
+            // grouped hand-over (see grouped_handover_ok): whole groups of four chunks, two groups at least
+            dc.grouped = elem == 4 && v.grouped_ok && !dc.embed && chunks % 4 == 0 && chunks >= 8 &&
+                         options().grouped != 0;
+            if (dc.grouped) dc.keep_bytes += 2 * pad256((size_t)rows * (chunks / 4) * v.low_size * elem);
+        }
         if (dc.resweep) dc.keep_bytes = (size_t)rows * v.sig_size * elem;
         return dc;
     }
@@ -2560,13 +2800,13 @@ static_assert(PSIG_GROUP < kDenseGroups, "group index out of range");
     case I:                                                                                                       \
         if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                      \
             return run_forward<T, D, N, P, PC, PS>(path, sig, shape, dc.fwd_chunks, bounds, keep, workspace,    \
-                                                   stream);                                                       \
+                                                   stream, dc.grouped);                                           \
         break;
 #define PSIG_CASE_BWD(I, D, N, P, PC, PS)                                                                          \
     case I:                                                                                                        \
         if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                       \
-            return run_backward<T, D, N, P, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape,       \
-                                                dc.bwd_chunks, bounds, kept, workspace, stream);                   \
+            return run_backward<T, D, N, P, PC, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape,   \
+                                                    dc.bwd_chunks, bounds, kept, workspace, stream, dc.grouped);   \
         break;
 
 template <int GROUP, typename T>

@@ -13,7 +13,7 @@ def pytest_configure(config):
 
 
 _OPTION_DEFAULTS = {"chunks": 0, "letter_bounds": 1, "logsig_scatter": 0, "batch_tile": 0, "embed_share": -1, "tiled": 1,
-                    "deep_fp64": 1}
+                    "deep_fp64": 1, "grouped": 1}
 
 
 @pytest.fixture

@@ -884,7 +884,8 @@ def test_letter_bounds_in_one_wave_blocks(ps, set_option, d, depth, chunks):
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
 @pytest.mark.parametrize("case", ["dense", "windows", "lyndon", "not_chunked", "per_word", "words_few_paths",
-                                  "words_many_paths", "words_windows"])
+                                  "words_many_paths", "words_windows", "groups_of_four", "three_groups",
+                                  "groups_windows", "groups_off"])
 def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case):
     """`compute_signature_keep` / `signature_backward_kept` (what the modules use when a gradient is wanted)
     against the reference's pair `compute_signature` / `signature_backward`: same signature, same dL/dpath.
@@ -906,6 +907,18 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
         d, depth, B, L = 8, 5, 2, 90
         kw["projection"] = ps.projections.lyndon(depth=depth, path_dim=d, full_levels=(1, 2, 3, 4))
         set_option("chunks", 3)
+    elif case in ("groups_of_four", "groups_off"):
+        d, depth, B, L = 4, 6, 3, 400       # fp32, a multiple of four chunks, eight and more: products within groups
+        set_option("chunks", 16)            # of four from the forward sweep, products of whole groups from a scan
+        if case == "groups_off":
+            set_option("grouped", 0)
+    elif case == "three_groups":
+        d, B, L = 4, 5, 333
+        set_option("chunks", 12)
+    elif case == "groups_windows":
+        d, B, L = 4, 3, 200
+        kw["windows"] = [(0, 200), (10, 150), (40, 42), (7, 7), (3, 199)]
+        set_option("chunks", 8)
     elif case == "not_chunked":
         d, B, L, chunked = 4, 3000, 20, False
     elif case == "per_word":
