@@ -96,7 +96,10 @@ int pathsig_sig_backward_noalloc(const void *path, const void *sig, const void *
  * from the signature of the row up to the chunk's right edge and from the signature of the rest of the row,
  * both below the top level (products of the chunks' own signatures).  The forward can write those two
  * arrays into `chunks`, and a backward that is given the same buffer skips the two launches that would
- * recompute them.  The per-word kernels hand over, in the same buffer, the
+ * recompute them.  (PATHSIG_F32 rows of eight and more chunks, a multiple of four, keep the factors of those
+ * products instead: every chunk's products with its neighbours inside its group of four chunks, and the products
+ * of the groups to the left and to the right of every group; the backward multiplies them as it starts a chunk.
+ * See the "grouped" option.)  The per-word kernels hand over, in the same buffer, the
  * prefix values of the words whose prefixes are not all part of the signature (the backward otherwise
  * rebuilds them with a forward sweep, as src/pathsig/backward/sig_backward_kernels.cu:134-157 does).
  * A word projection that is computed through a register-tiled shape which is swept in one piece (depth 2,
@@ -181,6 +184,10 @@ int pathsig_logsig_backward_kept(const void *logsig, const void *cache, const vo
  *                     path gradient at the end, unless it is a dense call of depth 9 cut into four time chunks or
  *                     more; 0 = in fp32 like any other call, two to three times as fast and off by up to 3.5e-5 of
  *                     the largest gradient at depth 12 (PATHSIG_NO_DEEP_FP64 sets 0)
+ *   "grouped"         1 (default) = a keeping PATHSIG_F32 forward whose rows are cut into eight or more time chunks,
+ *                     a multiple of four, keeps the chunk products by groups of four chunks (products within the
+ *                     groups and products of whole groups; pathsig_sig_chunks_bytes says how much), where the
+ *                     shape is compiled for it; 0 = products over all chunks of a row (PATHSIG_NO_GROUPED sets 0)
  * Returns PATHSIG_ERR_ARGUMENT for an unknown name or a value out of range.
  */
 int pathsig_set_option(const char *name, int64_t value);
