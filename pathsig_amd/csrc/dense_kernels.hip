@@ -936,7 +936,7 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             // (one set where two would not fit the register file beside the lane's state: fp64 over the widest
             // alphabets, whose sweep otherwise keeps part of its state in scratch memory)
             // (nor beside the hundred and more children of a lane over the widest alphabets)
-            constexpr bool kTwoSets = (sizeof(T) == 4 && D <= 64) ||
+            constexpr bool kTwoSets = (sizeof(T) == 4 && D <= 64 && !G::kLetterBlocks) ||
                                       (sizeof(T) == 8 && 2 * (G::kFwdSub + 2 * (KS * D + FQ * FK + P)) <= 384);
             if constexpr (kTwoSets) {
                 read(0, dxs0, dxp0, dxf0);
