@@ -856,6 +856,29 @@ def test_projection_through_dense_kernels_with_letter_bounds(ps, set_option, dty
         assert rel_err(got, plain) < TOL[dtype] and rel_err(grad, plain_grad) < TOL[dtype]
 
 
+@pytest.mark.parametrize("d,depth", [(2, 7), (3, 5), (3, 6), (3, 7), (4, 5), (4, 7), (5, 4), (5, 5), (6, 4), (6, 5),
+                                     (7, 4), (8, 4), (8, 5), (12, 4), (16, 4)])
+@pytest.mark.parametrize("chunks", [8, 12])
+def test_grouped_handover_across_shapes(ps, set_option, d, depth, chunks):
+    """fp32 rows of eight and more time chunks in whole groups of four: the keeping forward hands the chunk products
+    over by groups where the shape is compiled for it (the modules take the keeping pair).  Signature and gradient
+    against the checker, with chunks of unequal length and with windows, and against the run with the switch off."""
+    set_option("chunks", chunks)
+    B, L = 2, 16 * chunks + 5
+    path = brownian_path(B, L, d, seed=97) * (1.2 if depth < 7 else 0.8)
+    for windows in (None, [(0, L), (4, L - 3), (L // 3, L // 3 + 2)]):
+        want = TO.compute_signature(path, depth, windows=windows)
+        G = randn(tuple(want.shape), seed=98)
+        want_grad = TO.signature_vjp(path, G, depth, windows=windows)
+        got, grad = _run_sig(ps, path, depth, torch.float32, windows=windows, G=G)
+        assert rel_err(got, want) < TOL[torch.float32]
+        assert rel_err(grad, want_grad) < TOL[torch.float32]
+        set_option("grouped", 0)
+        plain, plain_grad = _run_sig(ps, path, depth, torch.float32, windows=windows, G=G)
+        set_option("grouped", 1)
+        assert torch.equal(got, plain) and rel_err(grad, plain_grad) < TOL[torch.float32]
+
+
 @pytest.mark.parametrize("d,depth", [(8, 5), (8, 4)])
 @pytest.mark.parametrize("chunks", [2, 3, 5])
 def test_letter_bounds_in_one_wave_blocks(ps, set_option, d, depth, chunks):
