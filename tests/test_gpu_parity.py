@@ -991,6 +991,13 @@ def test_forward_keeps_chunk_signatures_for_backward(ps, set_option, dtype, case
         again = torch.ops.pathsig.signature_backward_kept(x, sig, G, chunks, *args)
         assert rel_err(again, grad) < TOL[dtype]
         set_option("chunks", 5)
+    if case == "groups_of_four" and dtype == torch.float32:
+        # kept by groups, read back with the switch off: another size than the call would keep now, so left unread
+        set_option("grouped", 0)
+        assert chunks.numel() * chunks.element_size() > _load.lib().pathsig_sig_chunks_bytes(0, B, L, d, depth, sizes, 0)
+        again = torch.ops.pathsig.signature_backward_kept(x, sig, G, chunks, *args)
+        assert rel_err(again, grad) < TOL[dtype]
+        set_option("grouped", 1)
     checks = ("test_schema", "test_faketensor", "test_autograd_registration")
     if case in ("dense", "per_word") and dtype == torch.float64:
         torch.library.opcheck(torch.ops.pathsig.compute_signature_keep.default, (xg, *args), test_utils=checks)
