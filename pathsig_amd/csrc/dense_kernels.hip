@@ -962,9 +962,9 @@ __device__ __forceinline__ void dense_forward_body(const T *__restrict__ path, T
             // product c0 (x) .. (x) cj, group_suffix the product c(j+1) (x) .. (x) c3 (nothing for j = 3: the
             // identity), both below the top level; `out` receives the product of all four as before.  The products
             // that the block's result does not need run on the waves that would otherwise wait:
-            //   round 1   wave 0: c0 (x) c1          wave 2: c2 (x) c3
-            //   round 2   wave 0: (c0 c1) (x) (c2 c3)   wave 1: c1 (x) (c2 c3)   wave 3: (c0 c1) (x) c2   (the last two
-            //             below the top level)
+            //   first    wave 0: c0 (x) c1          wave 2: c2 (x) c3
+            //   then     wave 0: (c0 c1) (x) (c2 c3)   wave 1: c1 (x) (c2 c3)   wave 3: (c0 c1) (x) c2   (the last two
+            //            below the top level)
             constexpr int kLow = (int)G::kLowSize;
             const SubWords<D, P> sw(u);
             T *prefix_at = chunk_low + (row * chunks + c) * kLow;
