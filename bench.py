@@ -313,13 +313,14 @@ def run_config(name, dtype_name, args, with_graph, with_cpu, settle_ms):
         result["roofline_backward_call"] = {"bound": "valu", "achieved": ach, "peak": peak, "unit": "TFLOP/s",
                                             "frac": ach / peak, "traffic": None,
                                             "kernel": "signature backward call (all its launches)"}
-        # the dominant kernel alone: HIP events placed by the library around the reverse-sweep kernel
+        # the dominant kernel alone, as it runs inside the step (its backward starts from what the forward kept):
+        # HIP events placed by the library around the reverse-sweep kernel
         from pathsig_amd import _load
         lib = _load.lib()
         lib.pathsig_profile_enable(1)
         sweep = []
         for _ in range(args.steps):
-            torch.ops.pathsig.signature_backward(*args_b)
+            step()
             ms = float(lib.pathsig_profile_sweep_ms())
             if ms > 0:
                 sweep.append(ms)
