@@ -272,14 +272,19 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
         const T *sdense = (const T *)sig;
         const int64_t *top_codes = plan.code_off[depth] >= 0 ? codes + plan.code_off[depth] : nullptr;
         size_t used = 0;
+        bool prepared = false;
         if (dc.embed) {
             // upstream gradient scattered into a zeroed dense buffer.  The time-chunked backward rebuilds what it
             // reads of the dense signature; a shape that is swept in one piece reads the dense signature, which the
             // forward kept or which is swept again here
+            // (one launch clears the increment sums and the dense buffer behind them and, for a bounded call,
+            // computes the letter bounds where the backward looks for them: the head of its workspace)
             T *buf = (T *)extra;
-            used = dc.dense_bytes;
-            e = launch_fill_zero<T>(buf, (int64_t)(dc.dense_bytes / sizeof(T)), stream);
+            used = (dc.resweep ? 2 : 1) * dc.dense_bytes;
+            e = prepare_dense_backward<T>(dc, ginc, (int64_t)((inc_bytes + dc.dense_bytes) / sizeof(T)), top_codes,
+                                          plan.size[depth], extra + used, stream);
             if (e != hipSuccess) return launch_failed(e, "fill launch");
+            prepared = true;
             e = launch_scatter_columns<T>((const T *)grad_sig, buf, plan, d, codes, B * shape.W, stream);
             if (e != hipSuccess) return launch_failed(e, "scatter launch");
             gdense = buf;
@@ -294,13 +299,12 @@ int sig_backward_t(const void *path, const void *sig, const void *grad_sig, void
                     if (e != hipSuccess) return launch_failed(e, "dense forward launch");
                     sdense = again;
                 }
-                used = 2 * dc.dense_bytes;
             }
         }
         bool wrote_path = false;
         e = launch_dense_backward<T>((const T *)path, sdense, gdense, ginc, (T *)grad_path, &wrote_path, shape, dc,
                                      top_codes, plan.size[depth], dc.resweep ? (const T *)nullptr : (const T *)kept,
-                                     extra + used, stream);
+                                     extra + used, prepared, stream);
         if (e != hipSuccess) return launch_failed(e, "dense backward launch");
         if (wrote_path) return PATHSIG_OK;
     } else if (words_kernel || batch_wide) {

@@ -152,6 +152,24 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
                                  const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream);
+// ptr[0..n) = 0 by the threads tid, tid + stride, ..: 16-byte stores between the first and the last 16-byte
+// boundary of the buffer, single elements before and after
+template <typename T>
+__device__ __forceinline__ void zero_span(T *__restrict__ ptr, int64_t n, int64_t tid, int64_t stride) {
+    constexpr int VW = 16 / (int)sizeof(T);
+    typedef T V __attribute__((ext_vector_type(VW)));
+    int64_t head = (int64_t)(((16 - ((uintptr_t)ptr & 15)) & 15) / sizeof(T));
+    if (head > n) head = n;
+    const int64_t vecs = (n - head) / VW;
+    const int64_t tail_from = head + vecs * VW;
+    V *v = reinterpret_cast<V *>(ptr + head);
+    V zero;
+#pragma unroll
+    for (int k = 0; k < VW; ++k) zero[k] = T(0);
+    for (int64_t i = tid; i < vecs; i += stride) v[i] = zero;
+    if (tid < head) ptr[tid] = T(0);
+    if (tid < n - tail_from) ptr[tail_from + tid] = T(0);
+}
 // projected layout <- dense layout (gather) and dense layout += projected layout (scatter; dense zeroed before)
 template <typename T>
 hipError_t launch_gather_columns(const T *dense, T *out, const LevelPlan &plan, int64_t d, const int64_t *codes,

@@ -37,11 +37,19 @@ hipError_t launch_dense_forward(const T *path, T *sig, const SigShape &shape, co
                                 hipStream_t stream);
 // The backward fills grad_inc ([B, L-1, d] increment gradients), or, for time-chunked calls without windows,
 // writes grad_path ([B, L, d]) itself and reports that in *wrote_path.
+// prepared: prepare_dense_backward has run for this call (grad_inc is zero, the letter bounds of a bounded call
+// are at the head of `workspace`).
 template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                  bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
                                  const int64_t *top_codes, int64_t top_count, const T *kept, void *workspace,
-                                 hipStream_t stream);
+                                 bool prepared, hipStream_t stream);
+// One launch in front of the backward of an embedded projection, in place of three: clears zero[0..count) (the
+// per-increment sums and the dense gradient buffer behind them) and, for a bounded call, computes the letter
+// bounds into bounds_at (the head of the workspace that launch_dense_backward will be given).
+template <typename T>
+hipError_t prepare_dense_backward(const DenseChoice &dc, T *zero, int64_t count, const int64_t *top_codes,
+                                  int64_t top_count, void *bounds_at, hipStream_t stream);
 
 // The compiled shapes are dealt to kDenseGroups translation units (shape index modulo kDenseGroups); these are the
 // launch sequences of one group.  `bounds`: device array of letter bounds, or nullptr.
@@ -52,7 +60,8 @@ hipError_t launch_dense_forward_group(const T *path, T *sig, const SigShape &sha
 template <int GROUP, typename T>
 hipError_t launch_dense_backward_group(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                        bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
-                                       const int *bounds, const T *kept, void *workspace, hipStream_t stream);
+                                       const int *bounds, const T *kept, void *workspace, bool inc_cleared,
+                                       hipStream_t stream);
 
 // measurement hook: events around the reverse-sweep kernel of the last backward call (profile_bracket marks
 // the begin and the end of that kernel on its stream; a no-op while the hook is off)

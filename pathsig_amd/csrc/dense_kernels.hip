@@ -380,9 +380,8 @@ __device__ __forceinline__ void least_later_letter(C c, C d, int depth, int &fir
     first = (int)(c % d);
 }
 
-__global__ void __launch_bounds__(1024)
-    letter_bounds_kernel(const int64_t *__restrict__ codes, int64_t count, int d, int depth, bool narrow,
-                         int *__restrict__ bounds) {
+__device__ __forceinline__ void letter_bounds_block(const int64_t *__restrict__ codes, int64_t count, int d,
+                                                    int depth, bool narrow, int *__restrict__ bounds) {
     __shared__ int lo[16];
     if (threadIdx.x < 16) lo[threadIdx.x] = d;
     __syncthreads();
@@ -395,6 +394,24 @@ __global__ void __launch_bounds__(1024)
     }
     __syncthreads();
     if ((int)threadIdx.x < d) bounds[threadIdx.x] = lo[threadIdx.x];
+}
+
+__global__ void __launch_bounds__(1024)
+    letter_bounds_kernel(const int64_t *__restrict__ codes, int64_t count, int d, int depth, bool narrow,
+                         int *__restrict__ bounds) {
+    letter_bounds_block(codes, count, d, depth, narrow, bounds);
+}
+
+// The last block computes the letter bounds (when asked for: bounds != nullptr), the others clear ptr[0..n).
+template <typename T>
+__global__ void __launch_bounds__(1024)
+    zero_and_bounds_kernel(T *__restrict__ ptr, int64_t n, const int64_t *__restrict__ codes, int64_t count, int d,
+                           int depth, bool narrow, int *__restrict__ bounds) {
+    if (blockIdx.x + 1 == gridDim.x) {
+        if (bounds) letter_bounds_block(codes, count, d, depth, narrow, bounds);
+        return;
+    }
+    zero_span<T>(ptr, n, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)(gridDim.x - 1) * blockDim.x);
 }
 
 struct Span {
@@ -2513,7 +2530,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
 template <typename T, int D, int N, int P, int PC, int PS>
 hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path, bool *wrote_path,
                         const SigShape &shape, int chunks, const int *bounds, const T *kept, void *workspace,
-                        hipStream_t stream, bool grouped) {
+                        hipStream_t stream, bool grouped, bool inc_cleared) {
     using G = Geometry<D, N, P, sizeof(T)>;
     using GC = Geometry<D, N, PS>;
     constexpr bool kBoundsOk = LetterBounds<D, P>::kUsable && !G::kOnePiece;
@@ -2526,7 +2543,7 @@ hipError_t run_backward(const T *path, const T *sig, const T *grad_sig, T *grad_
     hipError_t e;
     // bounded sweeps exist for time-chunked calls only (every call that embeds a projection is chunked)
     if (bounds && (!kBoundsOk || chunks <= 1)) return hipErrorInvalidValue;
-    if (accumulate) {
+    if (accumulate && !inc_cleared) {
         e = launch_fill_zero<T>(grad_inc, shape.B * (shape.L - 1) * shape.d, stream);
         if (e != hipSuccess) return e;
     }
@@ -2769,17 +2786,36 @@ template <typename T>
 hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                  bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
                                  const int64_t *top_codes, int64_t top_count, const T *kept, void *workspace,
-                                 hipStream_t stream) {
+                                 bool prepared, hipStream_t stream) {
     if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
     if (kept && dc.keep_bytes == 0) return hipErrorInvalidValue;
-    const int *bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d,
-                                            kVariants[dc.variant].depth, &workspace, stream);
+    const int *bounds = nullptr;
+    if (prepared && dc.bounded) {
+        bounds = (const int *)workspace;
+        workspace = (unsigned char *)workspace + kBoundsBytes;
+    } else {
+        bounds = stage_letter_bounds(dc, top_codes, top_count, kVariants[dc.variant].d, kVariants[dc.variant].depth,
+                                     &workspace, stream);
+    }
     hipError_t e = hipErrorNotSupported;
     dispatch_group(dc.variant % kDenseGroups, [&](auto g) {
         e = launch_dense_backward_group<decltype(g)::value, T>(path, sig, grad_sig, grad_inc, grad_path, wrote_path,
-                                                               shape, dc, bounds, kept, workspace, stream);
+                                                               shape, dc, bounds, kept, workspace, prepared, stream);
     });
     return e;
+}
+
+template <typename T>
+hipError_t prepare_dense_backward(const DenseChoice &dc, T *zero, int64_t count, const int64_t *top_codes,
+                                  int64_t top_count, void *bounds_at, hipStream_t stream) {
+    if (dc.variant < 0 || dc.variant >= kNumVariants) return hipErrorNotSupported;
+    const int d = kVariants[dc.variant].d, depth = kVariants[dc.variant].depth;
+    const bool narrow = (double)depth * std::log2((double)d) < 32.0;
+    int64_t blocks = (count / (16 / (int64_t)sizeof(T)) + 1023) / 1024 + 1;  // one thread per 16-byte piece
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(zero_and_bounds_kernel<T>, dim3((unsigned)blocks + 1), dim3(1024), 0, stream, zero, count,
+                       top_codes, top_count, d, depth, narrow, dc.bounded ? (int *)bounds_at : (int *)nullptr);
+    return hipGetLastError();
 }
 
 #define PSIG_INSTANTIATE(T)                                                                                      \
@@ -2787,7 +2823,9 @@ hipError_t launch_dense_backward(const T *path, const T *sig, const T *grad_sig,
                                                 const int64_t *, int64_t, T *, void *, hipStream_t);             \
     template hipError_t launch_dense_backward<T>(const T *, const T *, const T *, T *, T *, bool *, const SigShape &, \
                                                  const DenseChoice &, const int64_t *, int64_t, const T *, void *,  \
-                                                 hipStream_t);
+                                                 bool, hipStream_t);                                                \
+    template hipError_t prepare_dense_backward<T>(const DenseChoice &, T *, int64_t, const int64_t *, int64_t,      \
+                                                  void *, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE
@@ -2806,7 +2844,8 @@ static_assert(PSIG_GROUP < kDenseGroups, "group index out of range");
     case I:                                                                                                        \
         if constexpr (I % kDenseGroups == PSIG_GROUP && shape_enabled(D, N))                                       \
             return run_backward<T, D, N, P, PC, PS>(path, sig, grad_sig, grad_inc, grad_path, wrote_path, shape,   \
-                                                    dc.bwd_chunks, bounds, kept, workspace, stream, dc.grouped);   \
+                                                    dc.bwd_chunks, bounds, kept, workspace, stream, dc.grouped,    \
+                                                    inc_cleared);                                                  \
         break;
 
 template <int GROUP, typename T>
@@ -2822,7 +2861,8 @@ hipError_t launch_dense_forward_group(const T *path, T *sig, const SigShape &sha
 template <int GROUP, typename T>
 hipError_t launch_dense_backward_group(const T *path, const T *sig, const T *grad_sig, T *grad_inc, T *grad_path,
                                        bool *wrote_path, const SigShape &shape, const DenseChoice &dc,
-                                       const int *bounds, const T *kept, void *workspace, hipStream_t stream) {
+                                       const int *bounds, const T *kept, void *workspace, bool inc_cleared,
+                                       hipStream_t stream) {
     switch (dc.variant) {
         PSIG_VARIANTS(PSIG_CASE_BWD)
         default: break;
@@ -2835,7 +2875,7 @@ hipError_t launch_dense_backward_group(const T *path, const T *sig, const T *gra
                                                                   const int *, T *, void *, hipStream_t);            \
     template hipError_t launch_dense_backward_group<PSIG_GROUP, T>(const T *, const T *, const T *, T *, T *, bool *,  \
                                                                    const SigShape &, const DenseChoice &, const int *, \
-                                                                   const T *, void *, hipStream_t);
+                                                                   const T *, void *, bool, hipStream_t);
 PSIG_INSTANTIATE(float)
 PSIG_INSTANTIATE(double)
 #undef PSIG_INSTANTIATE

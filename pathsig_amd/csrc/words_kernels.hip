@@ -311,24 +311,9 @@ __global__ void __launch_bounds__(kBwdBlock) words_backward_kernel(const T *__re
     }
 }
 
-// (16-byte stores between the first and the last 16-byte boundary of the buffer, single elements before and after)
 template <typename T>
 __global__ void fill_zero_kernel(T *__restrict__ ptr, int64_t n) {
-    constexpr int VW = 16 / (int)sizeof(T);
-    typedef T V __attribute__((ext_vector_type(VW)));
-    int64_t head = (int64_t)(((16 - ((uintptr_t)ptr & 15)) & 15) / sizeof(T));
-    if (head > n) head = n;
-    const int64_t vecs = (n - head) / VW;
-    const int64_t tail_from = head + vecs * VW;
-    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    V *v = reinterpret_cast<V *>(ptr + head);
-    V zero;
-#pragma unroll
-    for (int k = 0; k < VW; ++k) zero[k] = T(0);
-    for (int64_t i = tid; i < vecs; i += stride) v[i] = zero;
-    if (tid < head) ptr[tid] = T(0);
-    if (tid < n - tail_from) ptr[tail_from + tid] = T(0);
+    zero_span<T>(ptr, n, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
 }
 
 // dL/dx[t] = dL/d(dx[t-1]) - dL/d(dx[t]) with one-sided ends
