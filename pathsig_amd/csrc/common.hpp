@@ -152,6 +152,17 @@ hipError_t launch_batch_backward(const T *path, const T *sig, const T *grad_sig,
                                  const LevelPlan &plan, const int64_t *codes, hipStream_t stream);
 template <typename T>
 hipError_t launch_fill_zero(T *ptr, int64_t n, hipStream_t stream);
+// Grid of the kernels that run x over the columns of a row (256 threads to a block, a thread per column while
+// that keeps x below 2^16) and y over the rows, in strides of gridDim.y once the grid holds enough blocks to fill
+// the device several times: no thread divides an element index by the row length.
+inline dim3 columns_by_rows_grid(int64_t columns, int64_t rows) {
+    int64_t x = (columns + 255) / 256;
+    x = x < 1 ? 1 : (x > 65535 ? 65535 : x);
+    int64_t y = rows < 1 ? 1 : rows;
+    if (x * y > 16384) y = 16384 / x < 1 ? 1 : 16384 / x;
+    if (y > 65535) y = 65535;
+    return dim3((unsigned)x, (unsigned)y);
+}
 // ptr[0..n) = 0 by the threads tid, tid + stride, ..: 16-byte stores between the first and the last 16-byte
 // boundary of the buffer, single elements before and after
 template <typename T>

@@ -25,6 +25,7 @@
 //     v (or u) of a fixed length is a matrix-vector product over a dense level, so each output has one owner
 //     and nothing is atomic;
 //   * scatter form (any size): every word pushes its terms to its prefixes and suffixes with atomics.
+#include <cmath>
 #include <cstdlib>
 
 #include "common.hpp"
@@ -61,40 +62,50 @@ __device__ __forceinline__ constexpr T inv_factorial(int k) {
     return r;
 }
 
+// Dense columns (level offsets included) of every proper prefix and suffix of a word of DEG letters: pidx[k] its
+// first k letters, sidx[k] its last k letters, k = 1 .. DEG - 1.  One division per letter: the first k letters are
+// the first k + 1 without the last, and the last k are what the first DEG - k leave of the word.  IDX is uint32_t
+// when the codes of the level and the cache columns fit 32 bits (a 64-bit division by a run-time divisor is a
+// hundred instructions, and there would be 2 (DEG - 1) of them per word).
+template <typename IDX, int DEG>
+__device__ __forceinline__ void word_splits(IDX code, IDX d, IDX (&pidx)[DEG + 1], IDX (&sidx)[DEG + 1]) {
+    IDX first[DEG + 1];
+    first[DEG] = code;
+#pragma unroll
+    for (int k = DEG - 1; k >= 1; --k) first[k] = first[k + 1] / d;
+    IDX lo = 0, width = 1;
+#pragma unroll
+    for (int k = 1; k < DEG; ++k) {
+        width *= d;
+        pidx[k] = lo + first[k];
+        sidx[k] = lo + (code - first[DEG - k] * width);
+        lo += width;
+    }
+}
+
 // One level of one row.  STABLE: C is the cache of the Q form (entry k - 1 of a row holds Q_k; entry 0 the
 // log-signature itself), the right factors are log-signature values of the levels below, read from lg, and
 // lg receives the level.  Otherwise C is the power cache P of the reference, the right factors are signature
 // values, and lg is not touched.
-template <typename T, int DEG, bool STABLE>
+template <typename T, int DEG, bool STABLE, typename IDX>
 __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const HybridPlan &hp,
                                      const int64_t *__restrict__ top_words) {
     const int depth = hp.depth;
-    const uint64_t d = (uint64_t)hp.d;
+    const IDX d = (IDX)hp.d;
     const bool listed = (DEG == depth) && hp.top_is_list;
     const T *right = STABLE ? lg : s;
     // the blocks of one row (gridDim.y of them) share the words of the level
     for (int64_t i = (int64_t)blockIdx.y * (int)blockDim.x + threadIdx.x; i < hp.size[DEG]; i += (int64_t)gridDim.y * (int)blockDim.x) {
-        const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
+        const IDX code = listed ? (IDX)top_words[i] : (IDX)i;
         // dense column of every proper prefix, right factor of every proper suffix
-        uint64_t pidx[DEG + 1];
+        IDX pidx[DEG + 1], sidx[DEG + 1];
         T sufv[DEG + 1];
-        {
-            uint64_t div = 1;  // d^(DEG-k)
+        word_splits<IDX, DEG>(code, d, pidx, sidx);
 #pragma unroll
-            for (int k = 1; k < DEG; ++k) div *= d;
-            uint64_t lo = 0, width = 1;
-#pragma unroll
-            for (int k = 1; k < DEG; ++k) {
-                width *= d;
-                pidx[k] = lo + code / div;  // first k letters
-                sufv[k] = right[lo + code % width];  // last k letters
-                lo += width;
-                div /= d;
-            }
-        }
-        const uint64_t own = (uint64_t)(hp.off[DEG] + i);
+        for (int k = 1; k < DEG; ++k) sufv[k] = right[sidx[k]];
+        const IDX own = (IDX)(hp.off[DEG] + i);
         const T sw = s[own];
-        T *Cw = C + own * (uint64_t)depth;
+        T *Cw = C + own * (IDX)depth;
         // the Q form never reads the cache rows of the top level (nothing is longer than a top-level word), so
         // they are not written: for many rows the cache is most of what this kernel moves
         const bool keep_row = !STABLE || DEG < depth;
@@ -104,7 +115,7 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
         for (int m = 2; m <= DEG; ++m) {
             T pv = T(0);
 #pragma unroll
-            for (int k = m - 1; k < DEG; ++k) pv += C[pidx[k] * (uint64_t)depth + (uint64_t)(m - 2)] * sufv[DEG - k];
+            for (int k = m - 1; k < DEG; ++k) pv += C[pidx[k] * (IDX)depth + (IDX)(m - 2)] * sufv[DEG - k];
             if constexpr (STABLE) {
                 acc -= inv_factorial<T>(m) * pv;
                 qc -= inv_factorial<T>(m + 1) * pv;
@@ -129,7 +140,8 @@ __device__ void logsig_forward_level(const T *__restrict__ s, T *C, T *lg, const
 
 // Levels first..last of one row per blockIdx.x.  Several levels need one block per row (gridDim.y == 1: the
 // barrier between levels is a workgroup barrier); a single level may be shared by gridDim.y blocks.
-template <typename T, bool STABLE>
+// IDX: type of the column arithmetic (word_splits).
+template <typename T, bool STABLE, typename IDX>
 __global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__restrict__ sig, T *logsig, T *C,
                                                                    HybridPlan hp,
                                                                    const int64_t *__restrict__ top_words, int first,
@@ -141,7 +153,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_forward_kernel(const T *__re
     for (int deg = first; deg <= last; ++deg) {
         switch (deg) {
 #define PSIG_CASE(N) \
-    case N: logsig_forward_level<T, N, STABLE>(s, Cr, lg, hp, top_words); break;
+    case N: logsig_forward_level<T, N, STABLE, IDX>(s, Cr, lg, hp, top_words); break;
             PSIG_CASE(1) PSIG_CASE(2) PSIG_CASE(3) PSIG_CASE(4) PSIG_CASE(5) PSIG_CASE(6)
             PSIG_CASE(7) PSIG_CASE(8) PSIG_CASE(9) PSIG_CASE(10) PSIG_CASE(11) PSIG_CASE(12)
 #undef PSIG_CASE
@@ -194,20 +206,7 @@ __device__ void logsig_backward_level(const T *__restrict__ lgrow, const T *__re
     for (int64_t i = threadIdx.x; i < hp.size[DEG]; i += (int)blockDim.x) {
         const uint64_t code = listed ? (uint64_t)top_words[i] : (uint64_t)i;
         uint64_t pidx[DEG + 1], sidx[DEG + 1];
-        {
-            uint64_t div = 1;
-#pragma unroll
-            for (int k = 1; k < DEG; ++k) div *= d;
-            uint64_t lo = 0, width = 1;
-#pragma unroll
-            for (int k = 1; k < DEG; ++k) {
-                width *= d;
-                pidx[k] = lo + code / div;
-                sidx[k] = lo + code % width;
-                lo += width;
-                div /= d;
-            }
-        }
+        word_splits<uint64_t, DEG>(code, d, pidx, sidx);
         const uint64_t own = (uint64_t)(hp.off[DEG] + i);
         // a top-level word is nobody's prefix or suffix: nothing has been accumulated for it
         T lam = gl[own];
@@ -552,11 +551,12 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
 template <typename T>
 __global__ void scatter_top_kernel(const T *__restrict__ grad_logsig, T *__restrict__ dense, HybridPlan hp,
                                    const int64_t *__restrict__ top_words, int64_t rows, int64_t top_dense) {
-    const int64_t n = rows * hp.size[hp.depth];
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) {
-        const int64_t row = idx / hp.size[hp.depth], e = idx - row * hp.size[hp.depth];
-        atomicAdd(&dense[row * top_dense + top_words[e]], grad_logsig[row * hp.total + hp.off[hp.depth] + e]);
+    // grid: x over the listed words, y over the rows
+    const int64_t listed = hp.size[hp.depth];
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < listed; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t to = top_words[e], from = hp.off[hp.depth] + e;
+        for (int64_t row = blockIdx.y; row < rows; row += gridDim.y)
+            atomicAdd(&dense[row * top_dense + to], grad_logsig[row * hp.total + from]);
     }
 }
 
@@ -595,25 +595,35 @@ HybridPlan make_hybrid(int64_t d, int depth, int64_t top_size, const int64_t *to
 namespace {
 // one pass over all levels of all rows: the top level only reads the cache rows of the levels below it, so when
 // it is large it gets a launch of its own, with its words dealt out to several blocks per row
-template <typename T, bool STABLE>
-hipError_t forward_pass(const T *sig, T *logsig, T *C, const HybridPlan &hp, int64_t rows, int64_t top_size,
-                        const int64_t *top_words, hipStream_t stream) {
+template <typename T, bool STABLE, typename IDX>
+hipError_t forward_pass_as(const T *sig, T *logsig, T *C, const HybridPlan &hp, int64_t rows, int64_t top_size,
+                           const int64_t *top_words, hipStream_t stream) {
     const int depth = hp.depth;
     const int blk = logsig_block(hp.total, rows);
     int64_t slices = (top_size + 4 * blk - 1) / (4 * blk);
     if (slices > 16) slices = 16;
     if (depth < 2 || slices < 2) {
-        hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(blk), 0, stream, sig,
+        hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE, IDX>), dim3((unsigned)rows), dim3(blk), 0, stream, sig,
                            logsig, C, hp, top_words, 1, depth);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows), dim3(blk), 0, stream, sig, logsig,
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE, IDX>), dim3((unsigned)rows), dim3(blk), 0, stream, sig, logsig,
                        C, hp, top_words, 1, depth - 1);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE>), dim3((unsigned)rows, (unsigned)slices), dim3(blk), 0,
+    hipLaunchKernelGGL((logsig_forward_kernel<T, STABLE, IDX>), dim3((unsigned)rows, (unsigned)slices), dim3(blk), 0,
                        stream, sig, logsig, C, hp, top_words, depth, depth);
     return hipGetLastError();
+}
+
+template <typename T, bool STABLE>
+hipError_t forward_pass(const T *sig, T *logsig, T *C, const HybridPlan &hp, int64_t rows, int64_t top_size,
+                        const int64_t *top_words, hipStream_t stream) {
+    // 32-bit column arithmetic when every word code (below d^depth) and every cache column of a row fit
+    const double codes = std::pow((double)hp.d, (double)hp.depth);
+    const bool narrow = codes < 4294967296.0 && (double)hp.total * (double)hp.depth < 4294967296.0;
+    if (narrow) return forward_pass_as<T, STABLE, uint32_t>(sig, logsig, C, hp, rows, top_size, top_words, stream);
+    return forward_pass_as<T, STABLE, uint64_t>(sig, logsig, C, hp, rows, top_size, top_words, stream);
 }
 }  // namespace
 
@@ -690,10 +700,8 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                 if (e != hipSuccess) return e;
                 const int64_t n = rows * top_size;
                 if (n > 0) {
-                    int64_t blocks = (n + 255) / 256;
-                    if (blocks > 65536) blocks = 65536;
-                    hipLaunchKernelGGL(scatter_top_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad_logsig,
-                                       dense, hp, top_words, rows, lp.top_dense);
+                    hipLaunchKernelGGL(scatter_top_kernel<T>, columns_by_rows_grid(top_size, rows), dim3(256), 0, stream,
+                                       grad_logsig, dense, hp, top_words, rows, lp.top_dense);
                     e = hipGetLastError();
                     if (e != hipSuccess) return e;
                 }

@@ -319,20 +319,22 @@ __global__ void fill_zero_kernel(T *__restrict__ ptr, int64_t n) {
 // dL/dx[t] = dL/d(dx[t-1]) - dL/d(dx[t]) with one-sided ends
 // (reference: src/pathsig/backward/sig_backward_kernels.cu:347-377; 64-bit indices here)
 // (TI: type of the per-increment sums, fp64 behind the word-per-lane backward)
+// Grid: x over the L * d values of a path, y over the paths (no division by L * d; the one by d is a 32-bit
+// division when L * d fits 31 bits, and 64-bit divisions are a hundred instructions each).
 template <typename TI, typename T>
 __global__ void increments_to_path_kernel(const TI *__restrict__ ginc, T *__restrict__ gpath, int64_t B, int64_t L,
                                           int64_t d) {
-    const int64_t total = B * L * d;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t b = i / (L * d);
-        const int64_t rem = i - b * L * d;
-        const int64_t t = rem / d;
-        const int64_t a = rem - t * d;
-        const TI *g = ginc + b * (L - 1) * d + a;
-        const TI left = t > 0 ? g[(t - 1) * d] : TI(0);
-        const TI right = t < L - 1 ? g[t * d] : TI(0);
-        gpath[i] = (T)(left - right);
+    const int64_t per_path = L * d;
+    const bool narrow = per_path < (int64_t(1) << 31);
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < per_path; j += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = narrow ? (int64_t)((uint32_t)j / (uint32_t)d) : j / d;
+        const int64_t a = j - t * d;
+        for (int64_t b = blockIdx.y; b < B; b += gridDim.y) {
+            const TI *g = ginc + b * (L - 1) * d + a;
+            const TI left = t > 0 ? g[(t - 1) * d] : TI(0);
+            const TI right = t < L - 1 ? g[t * d] : TI(0);
+            gpath[b * per_path + j] = (T)(left - right);
+        }
     }
 }
 
@@ -357,12 +359,11 @@ __device__ __forceinline__ int64_t dense_column(const ColumnMap &m, const int64_
 template <typename T>
 __global__ void gather_columns_kernel(const T *__restrict__ dense, T *__restrict__ out, ColumnMap m,
                                       const int64_t *__restrict__ codes, int64_t rows) {
+    // grid: x over the projected columns, y over the rows (a thread looks its column up once)
     const int64_t width = m.out_off[m.depth + 1];
-    const int64_t total = rows * width;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t row = i / width;
-        out[i] = dense[row * m.dense_size + dense_column(m, codes, i - row * width)];
+    for (int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; col < width; col += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t from = dense_column(m, codes, col);
+        for (int64_t row = blockIdx.y; row < rows; row += gridDim.y) out[row * width + col] = dense[row * m.dense_size + from];
     }
 }
 
@@ -371,11 +372,10 @@ template <typename T>
 __global__ void scatter_columns_kernel(const T *__restrict__ grad, T *__restrict__ dense, ColumnMap m,
                                        const int64_t *__restrict__ codes, int64_t rows) {
     const int64_t width = m.out_off[m.depth + 1];
-    const int64_t total = rows * width;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t row = i / width;
-        atomicAdd(&dense[row * m.dense_size + dense_column(m, codes, i - row * width)], grad[i]);
+    for (int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; col < width; col += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t to = dense_column(m, codes, col);
+        for (int64_t row = blockIdx.y; row < rows; row += gridDim.y)
+            atomicAdd(&dense[row * m.dense_size + to], grad[row * width + col]);
     }
 }
 
@@ -468,10 +468,8 @@ hipError_t launch_increments_to_path(const TI *grad_inc, T *grad_path, int64_t B
                                      hipStream_t stream) {
     const int64_t n = B * L * d;
     if (n <= 0) return hipSuccess;
-    int64_t blocks = (n + 255) / 256;
-    if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL((increments_to_path_kernel<TI, T>), dim3((unsigned)blocks), dim3(256), 0, stream, grad_inc, grad_path,
-                       B, L, d);
+    const dim3 grid = columns_by_rows_grid(L * d, B);
+    hipLaunchKernelGGL((increments_to_path_kernel<TI, T>), grid, dim3(256), 0, stream, grad_inc, grad_path, B, L, d);
     return hipGetLastError();
 }
 
@@ -480,9 +478,7 @@ hipError_t launch_gather_columns(const T *dense, T *out, const LevelPlan &plan, 
                                  int64_t rows, hipStream_t stream) {
     const int64_t n = rows * plan.sig_size;
     if (n <= 0) return hipSuccess;
-    int64_t blocks = (n + 255) / 256;
-    if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(gather_columns_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, dense, out,
+    hipLaunchKernelGGL(gather_columns_kernel<T>, columns_by_rows_grid(plan.sig_size, rows), dim3(256), 0, stream, dense, out,
                        make_column_map(plan, d), codes, rows);
     return hipGetLastError();
 }
@@ -492,9 +488,7 @@ hipError_t launch_scatter_columns(const T *grad, T *dense, const LevelPlan &plan
                                   int64_t rows, hipStream_t stream) {
     const int64_t n = rows * plan.sig_size;
     if (n <= 0) return hipSuccess;
-    int64_t blocks = (n + 255) / 256;
-    if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(scatter_columns_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, grad, dense,
+    hipLaunchKernelGGL(scatter_columns_kernel<T>, columns_by_rows_grid(plan.sig_size, rows), dim3(256), 0, stream, grad, dense,
                        make_column_map(plan, d), codes, rows);
     return hipGetLastError();
 }
