@@ -411,7 +411,11 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_rows_kernel(
 // launch provides room for it (A_IN_LDS; the kernel is a chain of short dependent passes over `a`, so their
 // latency is what it costs), else in the workspace.  `R` ([lower columns], workspace) are the top-level sums of
 // logsig_gather_top_kernel, which has also stored the top-level part of the gradient in grad_sig.
-template <typename T, bool A_IN_LDS>
+// STAGED (with A_IN_LDS): everything else the passes read or update is brought to LDS in one burst of loads at the
+// start (the gradient of the levels below the top with the upstream gradient already added, the log-signature and
+// the cache rows of the levels 1 .. depth - 2), so that no pass waits for memory; the gradient goes back to memory
+// at the end.  For calls of a few hundred rows at most, where a row's latency is all there is.
+template <typename T, bool A_IN_LDS, bool STAGED = false>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ logsig,
                                                                   const T *__restrict__ cache,
                                                                   const T *__restrict__ grad_logsig, T *grad_sig,
@@ -425,10 +429,27 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     const T *gl = grad_logsig + row * hp.total;
     T *gs = grad_sig + row * hp.total;
     // the address space of `a` is fixed at compile time, so that its loads are LDS loads and not generic ones
+    static_assert(A_IN_LDS || !STAGED, "the staged form keeps `a` in LDS too");
     T *a;
     if constexpr (A_IN_LDS) a = reinterpret_cast<T *>(gather_smem);
     else a = a_all + row * hp.lower * N;
     const T *R = R_all + row * hp.lower;
+    const int64_t few = N >= 2 ? hp.off[N - 1] : 0;  // columns of the levels 1 .. N - 2
+    const T *lgsp, *Crp;
+    T *gsp;
+    if constexpr (STAGED) {
+        T *gs_l = a + hp.lower * N, *lgs_l = gs_l + hp.lower, *C_l = lgs_l + few;
+        for (int64_t i = threadIdx.x; i < few; i += (int)blockDim.x) lgs_l[i] = lgs[i];
+        for (int64_t i = threadIdx.x; i < few * N; i += (int)blockDim.x) C_l[i] = Cr[i];
+        for (int64_t i = threadIdx.x; i < hp.lower; i += (int)blockDim.x) gs_l[i] = gs[i] + gl[i];
+        lgsp = lgs_l;
+        Crp = C_l;
+        gsp = gs_l;
+    } else {
+        lgsp = lgs;
+        Crp = Cr;
+        gsp = gs;
+    }
     int64_t width[kMaxDepth + 1];  // d^k
     width[0] = 1;
     for (int k = 1; k <= N; ++k) width[k] = width[k - 1] * hp.d;
@@ -455,7 +476,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     const int BLK = (int)blockDim.x, tid = (int)threadIdx.x;
     for (int n = N - 1; n >= 1; --n) {
         T *an = a + hp.off[n] * N;
-        T *gsn = gs + hp.off[n];
+        T *gsn = gsp + hp.off[n];
         const int wn = (int)width[n];
         const int levels = N - 1 - n;  // levels between this one and the top
         if (levels > 0) {
@@ -476,7 +497,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
                         for (int i = 1; i <= levels; ++i) {
                             const int wi = (int)width[i];
                             const T *ap = a + (hp.off[n + i] + (int64_t)o * wi + part) * N + 1 + bi;
-                            const T *bp = lgs + hp.off[i] + part;
+                            const T *bp = lgsp + hp.off[i] + part;
                             for (int k = part; k < wi; k += parts) {
                                 acc += *ap * *bp;
                                 ap += (int64_t)parts * N;
@@ -511,7 +532,7 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
                         for (int j = 1; j <= levels; ++j) {
                             const int wj = (int)width[j];
                             const T *ap = a + (hp.off[n + j] + (int64_t)part * wn + o) * N + 1;
-                            const T *bp = Cr + (hp.off[j] + part) * N;
+                            const T *bp = Crp + (hp.off[j] + part) * N;
                             for (int k = part; k < wj; k += parts) {
                                 for (int m = 0; m < j; ++m) acc += ap[m] * bp[m];
                                 ap += (int64_t)parts * wn * N;
@@ -538,13 +559,15 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
         }
         // lam(w) = g(w) + a_1(w) + the sums above is the gradient of the word; a_k(w) -= lam(w) / k! for k >= 2
         for (int i = tid; i < wn; i += BLK) {
-            const T lam = gl[hp.off[n] + i] + an[i * N] + gsn[i];
+            const T lam = (STAGED ? T(0) : gl[hp.off[n] + i]) + an[i * N] + gsn[i];
             gsn[i] = lam;
             for (int k = 2; k <= n; ++k) an[i * N + k - 1] -= invf[k] * lam;
         }
         __threadfence_block();
         __syncthreads();
     }
+    if constexpr (STAGED)
+        for (int64_t i = threadIdx.x; i < hp.lower; i += (int)blockDim.x) gs[i] = gsp[i];
 }
 
 // dense[row][code of word e] += grad_logsig[row][top column e]; dense must be zero on entry
@@ -716,7 +739,16 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
         // the adjoint of the cache goes to LDS when a block's share of it fits beside the static arrays
         const size_t a_bytes = (size_t)hp.lower * (size_t)depth * sizeof(T);
         const bool a_in_lds = a_bytes <= 144 * 1024;
-        if (a_in_lds) {
+        const int64_t few = depth >= 2 ? hp.off[depth - 1] : 0;
+        const size_t staged_bytes = a_bytes + (size_t)(hp.lower + few * (1 + depth)) * sizeof(T);
+        if (a_in_lds && rows <= 512 && staged_bytes <= 150 * 1024) {
+            if (staged_bytes > 32 * 1024) {
+                e = allow_dynamic_lds<logsig_gather_kernel<T, true, true>>(staged_bytes);
+                if (e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL((logsig_gather_kernel<T, true, true>), dim3((unsigned)rows), dim3(blk), staged_bytes,
+                               stream, logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
+        } else if (a_in_lds) {
             if (a_bytes > 32 * 1024) {
                 e = allow_dynamic_lds<logsig_gather_kernel<T, true>>(a_bytes);
                 if (e != hipSuccess) return e;
