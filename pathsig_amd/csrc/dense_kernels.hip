@@ -1202,9 +1202,15 @@ __device__ __forceinline__ void combine_staged(const T *__restrict__ chunk_sig, 
     if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
 }
 
+// bounds (optional, not STAGED): the letter bounds of the sweep that made the chunk signatures.  A lane whose prefix
+// has a letter below the bound of its first letter after that first letter can only reach top-level words that the
+// sweep has left out: where the lanes sit on prefixes of length N - 1, it multiplies its chain and neither reads nor
+// writes anything above it (the row it leaves in `sig` is then undefined at those words, which no wanted word's
+// column maps to).
 template <typename T, int D, int N, int P, bool STAGED>
 __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
-    dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks) {
+    dense_combine_kernel(const T *__restrict__ chunk_sig, T *__restrict__ sig, int chunks,
+                         const int *__restrict__ bounds = nullptr) {
     using G = Geometry<D, N, P>;
     constexpr int kStage = STAGED ? CombineShape<T, D, N, P>::kStage : 4;
     __shared__ __align__(16) T sB[2][kStage];
@@ -1221,10 +1227,47 @@ __global__ void __launch_bounds__((Geometry<D, N, P>::kBlock))
         const T *rows = chunk_sig + row * chunks * G::kSigSize;
         T a[P + 1];
         T sub[G::kFwdSub];
-        load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
-        for (int c = 1; c < chunks; ++c)
-            apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
-        if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
+        // (only where the sub-trie of a lane is the top level alone: the levels below it are never left out)
+        bool above = true;  // the lane's sub-trie holds words that the sweep has not left out
+        if (bounds != nullptr && P == N - 1) {
+            const int lo = bounds[u[0]];
+#pragma unroll
+            for (int i = 1; i < P; ++i) above = above && u[i] >= lo;
+        }
+        if (above) {
+            load_state<T, D, P, N, G::kFwdSub>(rows, pu, active, a, sub);
+            for (int c = 1; c < chunks; ++c)
+                apply_right<T, D, P, N, G::kFwdSub>(a, sub, rows + (int64_t)c * G::kSigSize, sw);
+            if (active) store_state<T, D, P, N, G::kFwdSub>(sig + row * G::kSigSize, pu, a, sub);
+        } else {
+            // the chain alone (same operations as in load_state, apply_right and store_state)
+            int rest = 1;
+#pragma unroll
+            for (int j = P; j >= 1; --j) {
+                a[j] = active ? rows[G::level_off(j) + pu / rest] : T(0);
+                rest *= D;
+            }
+            a[0] = T(1);
+            for (int c = 1; c < chunks; ++c) {
+                const T *B = rows + (int64_t)c * G::kSigSize;
+#pragma unroll
+                for (int i = P; i >= 1; --i) {
+                    T acc = a[i];
+#pragma unroll
+                    for (int k = 0; k < i; ++k) acc = fmad<T>(a[k], B[G::level_off(i - k) + sw.code[k][i]], acc);
+                    a[i] = acc;
+                }
+            }
+            if (active) {
+                T *out = sig + row * G::kSigSize;
+                rest = 1;
+#pragma unroll
+                for (int j = P; j >= 1; --j) {
+                    out[G::level_off(j) + pu / rest] = a[j];
+                    rest *= D;
+                }
+            }
+        }
     }
 }
 
@@ -2522,7 +2565,7 @@ hipError_t run_forward(const T *path, T *sig, const SigShape &shape, int chunks,
                            (const T *)chunk_sig, sig, groups);
     else
         hipLaunchKernelGGL((dense_combine_kernel<T, D, N, PC, false>), dim3((unsigned)rows, (unsigned)GC::kUnitWaves),
-                           dim3(kWave), 0, stream, (const T *)chunk_sig, sig, groups);
+                           dim3(kWave), 0, stream, (const T *)chunk_sig, sig, groups, bounds);
     return hipGetLastError();
     }
 }
