@@ -275,6 +275,10 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
 // than threads the k range is split over `parts` threads per output and the partial sums meet in LDS
 // (`red`, one element per thread).  Lanes run along whichever of o and k is contiguous in A.  Ends with a
 // block barrier that also orders the stores in global memory for the next call.
+// When k is the contiguous index, nm = 1 and there are outputs enough to occupy the block that way, up to 64
+// consecutive lanes of a wave share an output instead, whatever the number of outputs: their loads are coalesced
+// (a thread that walks a row of its own makes every load of the wave touch 64 cache lines: measured 19 µs against
+// 7 for the same 128 KB), and the partial sums of eight outputs at a time meet through wave shuffles.
 struct MatvecShape {
     int64_t nb, no, nk, nm;   // batch, outputs, reduction length, inner terms
     int64_t ab, so, sk, sm;   // strides of A
@@ -292,6 +296,68 @@ __device__ void block_matvec(const T *A, const T *B, const MatvecShape &sh, T *r
     const int slots = (int)blockDim.x / parts;  // outputs worked on at once; >= outputs whenever parts > 1
     const bool k_fast = sh.sk < sh.so;
     const int tid = threadIdx.x;
+    if (k_fast && nm == 1 && (int)blockDim.x % kWave == 0) {
+        int lanes = 1;  // lanes of a wave that share an output
+        while (lanes * 2 <= kWave && lanes * 2 <= nk) lanes *= 2;
+        constexpr int kAtOnce = 8;
+        const int per_pass = (int)blockDim.x / lanes;  // outputs of one pass of the block
+        if (lanes >= 4 && outputs >= per_pass) {
+            const int at = tid % lanes, oloc = tid / lanes;
+            const int64_t astep = (int64_t)lanes * sh.sk, bstep = (int64_t)lanes * sh.sb;
+            for (int o0 = 0; o0 < outputs; o0 += per_pass * kAtOnce) {
+                T acc[kAtOnce];
+                int bi[kAtOnce], o[kAtOnce];
+#pragma unroll
+                for (int r = 0; r < kAtOnce; ++r) {
+                    const int oo = o0 + r * per_pass + oloc;
+                    const bool have = oo < outputs;
+                    bi[r] = have ? (sh.nb == 1 ? 0 : oo / no) : -1;
+                    o[r] = have ? oo - bi[r] * no : 0;
+                    acc[r] = T(0);
+                }
+                if (nk <= lanes) {
+                    // one term per lane: the loads of the eight outputs are in flight together
+                    T av[kAtOnce], bv[kAtOnce];
+#pragma unroll
+                    for (int r = 0; r < kAtOnce; ++r) {
+                        const bool have = bi[r] >= 0 && at < nk;
+                        const int b = have ? bi[r] : 0;
+                        av[r] = have ? A[(int64_t)b * sh.ab + (int64_t)o[r] * sh.so + (int64_t)at * sh.sk] : T(0);
+                        bv[r] = have ? B[(int64_t)b * sh.bb + (int64_t)at * sh.sb] : T(0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < kAtOnce; ++r) acc[r] = av[r] * bv[r];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < kAtOnce; ++r) {
+                        if (bi[r] < 0) continue;
+                        const T *ap = A + (int64_t)bi[r] * sh.ab + (int64_t)o[r] * sh.so + (int64_t)at * sh.sk;
+                        const T *bp = B + (int64_t)bi[r] * sh.bb + (int64_t)at * sh.sb;
+                        T sum = T(0);
+#pragma unroll 8
+                        for (int k = at; k < nk; k += lanes) {
+                            sum += *ap * *bp;
+                            ap += astep;
+                            bp += bstep;
+                        }
+                        acc[r] = sum;
+                    }
+                }
+                for (int off = lanes / 2; off >= 1; off /= 2) {
+#pragma unroll
+                    for (int r = 0; r < kAtOnce; ++r) acc[r] += __shfl_xor(acc[r], off);
+                }
+                if (at == 0) {
+#pragma unroll
+                    for (int r = 0; r < kAtOnce; ++r)
+                        if (bi[r] >= 0) store((int64_t)bi[r], (int64_t)o[r], acc[r]);
+                }
+            }
+            __threadfence_block();
+            __syncthreads();
+            return;
+        }
+    }
     const int part = k_fast ? tid % parts : tid / slots;
     const int oloc = k_fast ? tid / parts : tid % slots;
     const int64_t astep = (int64_t)parts * sh.sk, bstep = (int64_t)parts * sh.sb;
