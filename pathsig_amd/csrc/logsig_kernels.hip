@@ -269,6 +269,27 @@ __global__ void __launch_bounds__(kLogBlock) logsig_backward_kernel(const T *__r
 // ---------------------------------------------------------------------------------------------
 // gather form of the adjoint
 // ---------------------------------------------------------------------------------------------
+// use(i, load(i)) for i = threadIdx.x, threadIdx.x + blockDim.x, .. below count, with the loads of K rounds issued
+// before the first value is used: a loop that loads and uses one element per round waits for memory in every
+// round.  (The loads are unconditional, at a clamped index, so that the compiler can count them.)
+template <int K, typename Load, typename Use>
+__device__ __forceinline__ void batched_rounds(int64_t count, Load &&load, Use &&use) {
+    using V = decltype(load(int64_t(0)));
+    for (int64_t base = threadIdx.x; base < count; base += (int64_t)K * (int)blockDim.x) {
+        V v[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) {
+            const int64_t i = base + (int64_t)r * (int)blockDim.x;
+            v[r] = load(i < count ? i : count - 1);
+        }
+#pragma unroll
+        for (int r = 0; r < K; ++r) {
+            const int64_t i = base + (int64_t)r * (int)blockDim.x;
+            if (i < count) use(i, v[r]);
+        }
+    }
+}
+
 // A batch of matrix-vector products by all threads of the block:
 //     out[b][o] = sum_{k < nk} sum_{m < nm} A[b*ab + o*so + k*sk + m*sm] * B[b*bb + k*sb + m*sn]
 // for b < nb, o < no; store(b, o, value) runs once per output, in one thread.  When there are fewer outputs
@@ -414,12 +435,23 @@ template <typename T>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_top_kernel(const T *__restrict__ logsig,
                                                                       const T *__restrict__ cache,
                                                                       const T *__restrict__ gtop_all, T *grad_sig,
-                                                                      T *R_all, HybridPlan hp, int64_t top_dense) {
+                                                                      T *R_all, HybridPlan hp, int64_t top_dense,
+                                                                      const T *__restrict__ grad_logsig) {
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
     const int64_t row = blockIdx.x;
     const int j = (int)blockIdx.y + 1, i = N - j;
     const bool suffix_side = blockIdx.z == 1;
+    {
+        // the gradient of a top-level word is its upstream gradient: every block of the row copies a slice
+        const int64_t slices = 2 * (int64_t)gridDim.y, slice = 2 * (int64_t)blockIdx.y + blockIdx.z;
+        const int64_t per = (hp.size[N] + slices - 1) / slices;
+        const int64_t from = slice * per, to = from + per < hp.size[N] ? from + per : hp.size[N];
+        const T *gl = grad_logsig + row * hp.total + hp.off[N];
+        T *gs = grad_sig + row * hp.total + hp.off[N];
+        if (from < to)
+            batched_rounds<4>(to - from, [&](int64_t e) { return gl[from + e]; }, [&](int64_t e, T v) { gs[from + e] = v; });
+    }
     const T *lgs = logsig + row * hp.total;
     const T *gtop = gtop_all + row * top_dense;
     int64_t wi = 1, wj = 1;
@@ -485,7 +517,8 @@ template <typename T, bool A_IN_LDS, bool STAGED = false>
 __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__restrict__ logsig,
                                                                   const T *__restrict__ cache,
                                                                   const T *__restrict__ grad_logsig, T *grad_sig,
-                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp) {
+                                                                  T *a_all, const T *__restrict__ R_all, HybridPlan hp,
+                                                                  bool copy_top) {
     extern __shared__ __align__(16) unsigned char gather_smem[];
     __shared__ T red[kLogBlock];
     const int N = hp.depth;
@@ -505,9 +538,9 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
     T *gsp;
     if constexpr (STAGED) {
         T *gs_l = a + hp.lower * N, *lgs_l = gs_l + hp.lower, *C_l = lgs_l + few;
-        for (int64_t i = threadIdx.x; i < few; i += (int)blockDim.x) lgs_l[i] = lgs[i];
-        for (int64_t i = threadIdx.x; i < few * N; i += (int)blockDim.x) C_l[i] = Cr[i];
-        for (int64_t i = threadIdx.x; i < hp.lower; i += (int)blockDim.x) gs_l[i] = gs[i] + gl[i];
+        batched_rounds<4>(few, [&](int64_t i) { return lgs[i]; }, [&](int64_t i, T v) { lgs_l[i] = v; });
+        batched_rounds<8>(few * N, [&](int64_t i) { return Cr[i]; }, [&](int64_t i, T v) { C_l[i] = v; });
+        batched_rounds<8>(hp.lower, [&](int64_t i) { return gs[i] + gl[i]; }, [&](int64_t i, T v) { gs_l[i] = v; });
         lgsp = lgs_l;
         Crp = C_l;
         gsp = gs_l;
@@ -528,14 +561,15 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
         for (int k = 2; k <= N + 1; ++k) invf[k] = invf[k - 1] / T(k);
     }
     __syncthreads();
-    for (int n = 1; n < N; ++n) {
-        for (int64_t i = threadIdx.x; i < width[n]; i += (int)blockDim.x) {
-            const int64_t col = hp.off[n] + i;
-            const T r = R[col];
-            for (int m = 1; m <= N; ++m) a[col * N + m - 1] = m <= n ? -invf[m + 1] * r : T(0);
-        }
-    }
-    for (int64_t i = threadIdx.x; i < hp.size[N]; i += (int)blockDim.x) gs[hp.off[N] + i] = gl[hp.off[N] + i];
+    batched_rounds<8>(hp.lower, [&](int64_t col) { return R[col]; }, [&](int64_t col, T r) {
+        int n = 1;  // level of the column
+        while (n < N - 1 && col >= hp.off[n + 1]) ++n;
+        for (int m = 1; m <= N; ++m) a[col * N + m - 1] = m <= n ? -invf[m + 1] * r : T(0);
+    });
+    // (the launch over (row, split, side) has copied the top-level part already)
+    if (copy_top)
+        batched_rounds<8>(hp.size[N], [&](int64_t i) { return gl[hp.off[N] + i]; },
+                          [&](int64_t i, T v) { gs[hp.off[N] + i] = v; });
     __threadfence_block();
     __syncthreads();
 
@@ -548,12 +582,12 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
         if (levels > 0) {
             const int longest = (int)width[levels];
             // a_k(w) += sum_v a_{k+1}(w v) L(v), v over all those levels at once, k = 1..n (output = (k, w)).
-            // When there are fewer outputs than threads, `parts` threads share an output (lanes along v, which
-            // is contiguous in a) and their partial sums meet in LDS.
+            // When there are fewer outputs than threads, `parts` consecutive lanes of a wave share an output (lanes
+            // along v, which is contiguous in a) and their partial sums meet through wave shuffles.
             {
                 const int outputs = n * wn;
                 int parts = 1;
-                while (parts * 2 * outputs <= BLK && parts * 2 <= longest) parts *= 2;
+                while (parts * 2 * outputs <= BLK && parts * 2 <= longest && parts * 2 <= kWave) parts *= 2;
                 const int slots = BLK / parts, part = tid % parts, oloc = tid / parts;
                 for (int o0 = 0; o0 < outputs; o0 += slots) {
                     const int oo = o0 + oloc;
@@ -571,18 +605,8 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
                             }
                         }
                     }
-                    if (parts > 1) {
-                        red[tid] = acc;
-                        __syncthreads();
-                        if (part == 0 && oo < outputs) {
-                            T total = T(0);
-                            for (int q = 0; q < parts; ++q) total += red[oloc * parts + q];
-                            an[o * N + bi] += total;
-                        }
-                        __syncthreads();
-                    } else if (oo < outputs) {
-                        an[o * N + bi] += acc;
-                    }
+                    for (int off = parts / 2; off >= 1; off /= 2) acc += __shfl_xor(acc, off);
+                    if (part == 0 && oo < outputs) an[o * N + bi] += acc;
                 }
             }
             // gradient(w) += sum_u sum_{k=2}^{|u|+1} a_k(u w) Q_{k-1}(u), u over the same levels (output = w; lanes
@@ -607,14 +631,27 @@ __global__ void __launch_bounds__(kLogBlock) logsig_gather_kernel(const T *__res
                         }
                     }
                     if (parts > 1) {
-                        red[tid] = acc;
-                        __syncthreads();
-                        if (part == 0 && o < wn) {
-                            T total = T(0);
-                            for (int q = 0; q < parts; ++q) total += red[q * slots + oloc];
-                            gsn[o] += total;
+                        // the parts of an output are `slots` threads apart: those inside a wave meet through
+                        // shuffles, the waves' sums in LDS
+                        int left = parts, stride = slots;  // partial sums still apart, and by how many threads
+                        if (slots < kWave && BLK % kWave == 0) {
+                            for (int off = kWave / 2; off >= slots; off /= 2) acc += __shfl_xor(acc, off);
+                            const int in_wave = kWave / slots < parts ? kWave / slots : parts;
+                            left = parts / in_wave;
+                            stride = kWave;
                         }
-                        __syncthreads();
+                        if (left > 1) {
+                            red[tid] = acc;
+                            __syncthreads();
+                            if (part == 0 && o < wn) {
+                                T total = T(0);
+                                for (int q = 0; q < left; ++q) total += red[q * stride + oloc];
+                                gsn[o] += total;
+                            }
+                            __syncthreads();
+                        } else if (part == 0 && o < wn) {
+                            gsn[o] += acc;
+                        }
                     } else if (o < wn) {
                         gsn[o] += acc;
                     }
@@ -773,6 +810,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
         // top-level products: with many rows of a small layout one block per row with the row's dense top-level
         // gradient in LDS; else one block per (row, split, side) over a dense copy of that gradient in memory
         const size_t top_bytes = (size_t)lp.top_dense * sizeof(T);
+        bool copy_top = true;  // the lower-level kernel copies the top-level part of the gradient
         if (rows >= 256 && top_bytes <= 64 * 1024) {
             if (top_bytes > 32 * 1024) {
                 e = allow_dynamic_lds<logsig_gather_top_rows_kernel<T>>(top_bytes);
@@ -781,6 +819,7 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
             hipLaunchKernelGGL(logsig_gather_top_rows_kernel<T>, dim3((unsigned)rows), dim3(blk), top_bytes, stream,
                                logsig, cache, grad_logsig, grad_sig, R, hp, top_words, lp.top_dense);
         } else {
+            copy_top = false;  // (the launch over (row, split, side) does)
             const T *gtop = grad_logsig + hp.off[depth];
             int64_t top_stride = hp.total;  // dense top level: read in place, row stride of the gradient
             if (lp.top_elems > 0) {
@@ -798,7 +837,8 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                 top_stride = lp.top_dense;
             }
             hipLaunchKernelGGL(logsig_gather_top_kernel<T>, dim3((unsigned)rows, (unsigned)(depth - 1), 2),
-                               dim3(kLogBlock), 0, stream, logsig, cache, gtop, grad_sig, R, hp, top_stride);
+                               dim3(kLogBlock), 0, stream, logsig, cache, gtop, grad_sig, R, hp, top_stride,
+                               grad_logsig);
         }
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -813,17 +853,17 @@ hipError_t launch_logsig_backward(const T *logsig, const T *cache, const T *grad
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL((logsig_gather_kernel<T, true, true>), dim3((unsigned)rows), dim3(blk), staged_bytes,
-                               stream, logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
+                               stream, logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp, copy_top);
         } else if (a_in_lds) {
             if (a_bytes > 32 * 1024) {
                 e = allow_dynamic_lds<logsig_gather_kernel<T, true>>(a_bytes);
                 if (e != hipSuccess) return e;
             }
             hipLaunchKernelGGL((logsig_gather_kernel<T, true>), dim3((unsigned)rows), dim3(blk), a_bytes, stream,
-                               logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
+                               logsig, cache, grad_logsig, grad_sig, gradP, (const T *)R, hp, copy_top);
         } else {
             hipLaunchKernelGGL((logsig_gather_kernel<T, false>), dim3((unsigned)rows), dim3(blk), 0, stream, logsig,
-                               cache, grad_logsig, grad_sig, gradP, (const T *)R, hp);
+                               cache, grad_logsig, grad_sig, gradP, (const T *)R, hp, copy_top);
         }
         return hipGetLastError();
     }
